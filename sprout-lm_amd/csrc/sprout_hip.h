@@ -155,6 +155,61 @@ int sp_sample_static(void* stream, const float* logits, const float* temperature
                      const int32_t* counter, int32_t* out, int R, int V);
 int sp_sample_static_max_floats();
 
+// Layer norm without bias: out[r, :] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w, x float32 [*, H], rows as in
+// sp_rmsnorm.
+int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, float eps,
+                 int out_dtype, void* out, int R, int H);
+
+// residual[t, :] = table[tokens[t], :] + pairs[row, :] with row = (previous * mul_prev + tokens[t] * mul_cur) mod buckets,
+// and row `buckets` (the table's last) at position 0.  The token before a step's first token of a sequence is read
+// from last_token[state_slots[seq]] (int32, one entry per state slot), where the step's last token of the sequence
+// is left for the next step.
+int sp_embed_bigram(void* stream, int table_dtype, const void* table, const void* pairs, const int32_t* tokens,
+                    const int32_t* positions, const int32_t* q_start, const int32_t* q_len, const int32_t* seq_of_token,
+                    const int32_t* state_slots, int32_t* last_token, float* residual, int T, int H, int V, int buckets,
+                    int mul_prev, int mul_cur);
+
+// Attention over a latent, between the input projections and the attention kernel.  A row of proj holds per head
+// [dim unrotated, rot rotated] query numbers from column q_off on, and at dkv_off the latent (rank numbers) and
+// one rotated key part (rot numbers).  Writes, per token: the RMS-normed latent and the turned key part as the key
+// [rank + rot] of the one key/value head at slot_mapping[t] (null: nothing is cached), the latent as the value
+// (the value pool's last rot columns are left alone), and every head's turned query part into
+// q_out[t, head, rank : rank + rot] (rows of heads * (rank + rot)).  The first rot_dims numbers of a rotated part
+// turn, (2i, 2i + 1) together, by positions[t] * freq[i] with cosine and sine times `magnitude`; exact != 0: the
+// angle and its cosine and sine in float64.
+int sp_latent_prepare(void* stream, int dtype, const void* proj, int proj_stride, int q_off, int heads, int dim, int rot,
+                      int dkv_off, int rank, int norm_w_dtype, const void* norm_w, float eps, const int32_t* positions,
+                      const double* freq, int rot_dims, float magnitude, int exact, const int32_t* slot_mapping,
+                      void* k_pool, void* v_pool, int page_size, int num_pages, void* q_out, int T);
+
+// Per-head products: out[t, h * out_head_stride + n] = sum_k a[t, h * a_head_stride + k] * w[h][n][k]
+// (w [heads, N, K]; rows of a and out are a_stride and out_stride apart; all three of `dtype`), times
+// sigmoid(gate[t * gate_stride + h]) where gate is given.
+int sp_head_gemm(void* stream, int dtype, const void* a, long long a_stride, long long a_head_stride, const void* w,
+                 void* out, long long out_stride, long long out_head_stride, const void* gate, long long gate_stride,
+                 int T, int heads, int N, int K);
+
+// A feed-forward with experts.  sp_route_topk: ids, weights [T, top] = the `top` largest of each token's `experts`
+// float32 logits (falling, the lowest index wins a tie) and the softmax over those alone.  sp_route_sort orders the
+// T * top pairs by expert: row_of_pair and its inverse pair_of_row, and tiles [n][3] = (expert, first row, rows) of at
+// most tile_rows rows with n in *n_tiles (at most sp_route_max_tiles(pairs, experts, tile_rows)).  sp_expert_gate_up:
+// out[row, :] = act(x[token] . w[e][:inner]^T) * (x[token] . w[e][inner:]^T) for the rows of every tile (token =
+// pair_of_row[row] / top; w [experts, 2 inner, K]).  sp_expert_down: out[row, :] = act[row] . w[e]^T in float32
+// (w [experts, hidden, inner]).  sp_route_combine: residual[t] += sum_k weights[t, k] * y[row_of_pair[t * top + k]].
+// sp_group_tile_rows(): the tile_rows that the grouped products take.
+int sp_group_tile_rows();
+int sp_route_topk(void* stream, const float* logits, int32_t* ids, float* weights, int T, int experts, int top);
+int sp_route_max_tiles(int pairs, int experts, int tile_rows);
+int sp_route_sort(void* stream, const int32_t* ids, int pairs, int experts, int tile_rows, int32_t* row_of_pair,
+                  int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
+int sp_expert_gate_up(void* stream, int dtype, const void* x, const void* w, const int32_t* tiles, const int32_t* n_tiles,
+                      int max_tiles, const int32_t* pair_of_row, int top, void* out, int T, int experts, int inner, int K,
+                      int activation);
+int sp_expert_down(void* stream, int dtype, const void* act, const void* w, const int32_t* tiles, const int32_t* n_tiles,
+                   int max_tiles, float* out, int rows, int experts, int hidden, int inner);
+int sp_route_combine(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,
+                     float* residual, int T, int H);
+
 // Probes for the benchmark's report, not used by the engine: a kernel that only reads `bytes` of `data` (16-byte
 // loads from `blocks` blocks of 256 threads), and one that only multiplies on the matrix cores (`blocks` blocks of four waves,
 // `iterations` x 4 independent 32x32x16 bfloat16 products a wave; *flops receives the operations of one launch).

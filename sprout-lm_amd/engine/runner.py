@@ -279,7 +279,17 @@ class ModelRunner:
         T, H = ctx.n_tokens, self.hidden_size
         with ops.stream_scope():       # one stream lookup for the step's launches
             residual = ctx.buffer("residual", (T, H), torch.float32)
-            self.parts.embedding.forward(ctx, ctx.token_ids, residual)
+            if self.parts.embedding_slot is None:
+                self.parts.embedding.forward(ctx, ctx.token_ids, residual)
+            else:       # an embedding that keeps something per request (the token before a step's first one)
+                kind, g, index = self.cache.slot_location[self.parts.embedding_slot]
+                if kind == "state":
+                    kept = CacheSlotView(True, state=self.cache.state_groups[g].data[index])
+                else:
+                    group = self.cache.groups[g]
+                    kept = CacheSlotView(True, k=group.k[index], v=group.v[index], block_tables=ctx.group_tables[g],
+                                         slot_mapping=ctx.group_slots[g], page_size=group.page_tokens)
+                self.parts.embedding.forward(ctx, ctx.token_ids, residual, kept)
             for i, call in enumerate(self.plan.schedule):
                 self.parts.blocks[call.layer].forward(ctx, residual, self._slot_views(ctx, i))
             n = ctx.n_logits

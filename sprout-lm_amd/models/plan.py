@@ -66,6 +66,9 @@ class ModelPlan:
     # state of fixed size, which is no function of pages and would have to be rebuilt with them; an architecture
     # that knows better (a state it can snapshot at page edges, pages that depend on more than the tokens) says so.
     prefix_sharing: bool | None = None
+    # The cache slot of what the embedding keeps between steps (a part that reads the token before a step's first
+    # one keeps it per request); None where the embedding keeps nothing.
+    embedding_slot: int | None = None
 
     def instantiate(self) -> "ModelParts":
         return ModelParts(self)
@@ -125,6 +128,14 @@ class ModelParts:
                 if not writes and slots.get(slot) != needs[key]:
                     raise ValueError(f"Layer {call.layer} reads cache slot {slot}, which no call writes with the "
                                      f"same shape.")
+        needed = self.embedding.cache_spec()
+        if (needed is None) != (plan.embedding_slot is None):
+            raise ValueError("The plan must name a cache slot for the embedding exactly if the embedding keeps something.")
+        if needed is not None:
+            if plan.embedding_slot in slots:
+                raise ValueError(f"Cache slot {plan.embedding_slot} of the embedding is also written by a layer.")
+            slots[plan.embedding_slot] = needed
+        self.embedding_slot = plan.embedding_slot
         if sorted(slots) != list(range(len(slots))):
             raise ValueError("Cache slots of the run order must be numbered 0..n-1 without gaps.")
         self.cache_slot_specs = [slots[i] for i in range(len(slots))]

@@ -61,7 +61,8 @@ def _ptr(t):
 
 # Variants of an operation that a part may ask for, as the C interface numbers them.  Only the listed ones have
 # kernels; anything else is refused (KernelError) before a launch.
-ROTARY_PAIRINGS = {"halves": 0}          # dimension d turns with d + rotary_dim / 2 ("neox")
+ROTARY_PAIRINGS = {"halves": 0}          # dimension d turns with d + rotary_dim / 2 ("neox"); the latent mixer's own
+                                         # kernel (latent_prepare) turns neighbours (2i, 2i + 1)
 GATE_ACTIVATIONS = {"silu": 0}
 SCORE_STAGES = {"scaled_dot": 0}         # what stands between q . k and the softmax: the scale and nothing else
 MAX_HEAD_DIM = 512                       # the largest head size any attention kernel takes
@@ -119,6 +120,162 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
         raise KernelError("rmsnorm: fewer input rows than output rows")
     check(library().sp_rmsnorm(_stream(), x.data_ptr(), _ptr(rows), _code(weight, "norm weight"), weight.data_ptr(),
                                float(eps), _code(out, "norm output"), out.data_ptr(), R, H))
+
+
+def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+    """out[r] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight of x[rows[r]] or x[r]; x is float32."""
+    _gpu(x, "norm input"); _gpu(weight, "norm weight"); _gpu(out, "norm output")
+    R, H = out.shape
+    if x.dtype != torch.float32 or x.shape[1] != H or weight.numel() != H:
+        raise KernelError(f"layernorm: shapes do not fit: x {tuple(x.shape)} {x.dtype}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    if rows is not None:
+        _ints(rows, R, "norm rows")
+    elif x.shape[0] < R:
+        raise KernelError("layernorm: fewer input rows than output rows")
+    check(library().sp_layernorm(_stream(), x.data_ptr(), _ptr(rows), _code(weight, "norm weight"), weight.data_ptr(),
+                                 float(eps), _code(out, "norm output"), out.data_ptr(), R, H))
+
+
+def embed_bigram(table: torch.Tensor, pairs: torch.Tensor, tokens, positions, q_start, q_len, seq_of_token, state_slots,
+                 last_token: torch.Tensor, residual: torch.Tensor, n_seqs: int, buckets: int, mul_prev: int, mul_cur: int) -> None:
+    """residual[t] = table[tokens[t]] + pairs[(previous * mul_prev + tokens[t] * mul_cur) % buckets] (row `buckets` at
+    position 0) as float32.  `last_token` (int32, one entry per state slot) carries a sequence's last token from step
+    to step."""
+    _gpu(table, "embedding table"); _gpu(pairs, "pair table"); _gpu(residual, "residual"); _gpu(last_token, "last tokens")
+    T = residual.shape[0]
+    V, H = table.shape
+    if residual.dtype != torch.float32 or residual.shape[1] != H:
+        raise KernelError(f"embed_bigram: residual must be float32 [T, {H}], got {residual.dtype} {tuple(residual.shape)}")
+    if tuple(pairs.shape) != (buckets + 1, H) or pairs.dtype != table.dtype:
+        raise KernelError(f"embed_bigram: the pair table must be [{buckets + 1}, {H}] {table.dtype}, got {tuple(pairs.shape)} {pairs.dtype}")
+    if last_token.dtype != torch.int32:
+        raise KernelError("embed_bigram: last tokens must be int32")
+    for t, n, what in ((tokens, T, "tokens"), (positions, T, "positions"), (seq_of_token, T, "seq_of_token"),
+                       (q_start, n_seqs, "q_start"), (q_len, n_seqs, "q_len"), (state_slots, n_seqs, "state_slots")):
+        _ints(t, n, what)
+    check(library().sp_embed_bigram(_stream(), _code(table, "embedding table"), table.data_ptr(), pairs.data_ptr(),
+                                    tokens.data_ptr(), positions.data_ptr(), q_start.data_ptr(), q_len.data_ptr(),
+                                    seq_of_token.data_ptr(), state_slots.data_ptr(), last_token.data_ptr(),
+                                    residual.data_ptr(), T, H, V, int(buckets), int(mul_prev), int(mul_cur)))
+
+
+def latent_prepare(proj: torch.Tensor, q_off: int, heads: int, dim: int, rot: int, dkv_off: int, rank: int,
+                   norm_weight: torch.Tensor, eps: float, positions, freq: torch.Tensor, rot_dims: int, magnitude: float,
+                   slot_mapping, k_pool, v_pool, q_out: torch.Tensor) -> None:
+    """From a row of projections: the normed latent and the turned shared key part into the pools (keys
+    [pages, 1, page, rank + rot], values [pages, 1, rank + rot, page], whose last rot columns are left alone), and
+    every head's turned query part into q_out[t, head, rank:] (see sprout_hip.h).  Float32 rows turn by float64 angles."""
+    _gpu(proj, "projections"); _gpu(norm_weight, "latent norm weight"); _gpu(q_out, "latent queries"); _gpu(freq, "frequencies")
+    T, stride = proj.shape
+    width = rank + rot
+    if tuple(q_out.shape) != (T, heads * width) or q_out.dtype != proj.dtype:
+        raise KernelError(f"latent_prepare: queries must be [{T}, {heads * width}] {proj.dtype}, got {tuple(q_out.shape)} {q_out.dtype}")
+    if norm_weight.numel() != rank or freq.dtype != torch.float64 or freq.numel() < rot_dims // 2:
+        raise KernelError("latent_prepare: the norm weight must hold rank numbers and freq rot_dims / 2 float64 numbers")
+    _ints(positions, T, "positions")
+    page_size = num_pages = 0
+    if slot_mapping is not None:
+        _ints(slot_mapping, T, "slot_mapping")
+        num_pages, page_size = _check_pools(k_pool, v_pool, 1, width, proj.dtype, "latent_prepare")
+    check(library().sp_latent_prepare(_stream(), _code(proj, "projections"), proj.data_ptr(), stride, q_off, heads, dim, rot,
+                                      dkv_off, rank, _code(norm_weight, "latent norm weight"), norm_weight.data_ptr(),
+                                      float(eps), positions.data_ptr(), freq.data_ptr(), rot_dims, float(magnitude),
+                                      int(proj.dtype == torch.float32), _ptr(slot_mapping), _ptr(k_pool), _ptr(v_pool),
+                                      page_size, num_pages, q_out.data_ptr(), T))
+
+
+def head_gemm(a: torch.Tensor, a_offset: int, a_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_offset: int,
+              out_head_stride: int, gate: torch.Tensor | None = None, gate_offset: int = 0) -> None:
+    """Per head h: out[t, out_offset + h * out_head_stride + n] = sum_k a[t, a_offset + h * a_head_stride + k] * w[h, n, k],
+    times sigmoid(gate[t, gate_offset + h]) where `gate` is given.  w [heads, N, K]; a, w, out (and gate) of one dtype."""
+    _gpu(a, "head product input"); _gpu(w, "head product weight"); _gpu(out, "head product output")
+    heads, N, K = w.shape
+    T = out.shape[0]
+    if a.dtype != w.dtype or out.dtype != w.dtype or a.shape[0] < T:
+        raise KernelError(f"head_gemm: dtypes or rows do not fit: a {a.dtype} {tuple(a.shape)}, w {w.dtype}, out {out.dtype} {tuple(out.shape)}")
+    if (a_offset < 0 or a_offset + (heads - 1) * a_head_stride + K > a.shape[1]
+            or out_offset < 0 or out_offset + (heads - 1) * out_head_stride + N > out.shape[1]):
+        raise KernelError(f"head_gemm: {heads} heads of K={K}, N={N} do not fit rows of {a.shape[1]} and {out.shape[1]}")
+    size = a.element_size()
+    gate_ptr, gate_stride = None, 0
+    if gate is not None:
+        _gpu(gate, "head gate")
+        if gate.dtype != w.dtype or gate.shape[0] < T or gate_offset < 0 or gate_offset + heads > gate.shape[1]:
+            raise KernelError("head_gemm: the gate does not hold a number per token and head")
+        gate_ptr, gate_stride = gate.data_ptr() + gate_offset * size, gate.shape[1]
+    check(library().sp_head_gemm(_stream(), _code(w, "head product weight"), a.data_ptr() + a_offset * size, a.shape[1],
+                                 a_head_stride, w.data_ptr(), out.data_ptr() + out_offset * size, out.shape[1],
+                                 out_head_stride, gate_ptr, gate_stride, T, heads, N, K))
+
+
+def group_tile_rows() -> int:
+    return library().sp_group_tile_rows()
+
+
+def route_max_tiles(pairs: int, experts: int) -> int:
+    return library().sp_route_max_tiles(pairs, experts, group_tile_rows())
+
+
+def route_topk(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """ids, weights [T, top] = the top largest logits of every row (falling; the lowest index wins a tie) and the
+    softmax over those alone."""
+    _gpu(logits, "router logits"); _gpu(ids, "chosen experts"); _gpu(weights, "expert weights")
+    T, E = logits.shape
+    top = ids.shape[1]
+    if logits.dtype != torch.float32 or ids.dtype != torch.int32 or weights.dtype != torch.float32 or \
+            tuple(ids.shape) != (T, top) or tuple(weights.shape) != (T, top) or not 0 < top <= E:
+        raise KernelError("route_topk: float32 logits [T, E], int32 ids and float32 weights [T, top] expected")
+    check(library().sp_route_topk(_stream(), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E, top))
+
+
+def route_sort(ids: torch.Tensor, experts: int, row_of_pair, pair_of_row, tiles, n_tiles) -> None:
+    """Orders the (token, choice) pairs by expert for the grouped products (see sprout_hip.h)."""
+    pairs = ids.numel()
+    _ints(ids, pairs, "chosen experts"); _ints(row_of_pair, pairs, "row_of_pair"); _ints(pair_of_row, pairs, "pair_of_row")
+    _ints(tiles, 3 * route_max_tiles(pairs, experts), "expert tiles"); _ints(n_tiles, 1, "tile count")
+    check(library().sp_route_sort(_stream(), ids.data_ptr(), pairs, experts, group_tile_rows(), row_of_pair.data_ptr(),
+                                  pair_of_row.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr()))
+
+
+def expert_gate_up(x: torch.Tensor, w: torch.Tensor, tiles, n_tiles, pair_of_row, top: int, out: torch.Tensor,
+                   activation: str = "silu") -> None:
+    """out[row] = act(x[token] . w[e, :I]^T) * (x[token] . w[e, I:]^T) for every sorted row (w [experts, 2 I, K])."""
+    _gpu(x, "expert input"); _gpu(w, "expert gate/up weights"); _gpu(out, "expert activations")
+    T, K = x.shape
+    E, two_i, _ = w.shape
+    if w.shape[2] != K or two_i % 2 or tuple(out.shape) != (T * top, two_i // 2) or not (x.dtype == w.dtype == out.dtype):
+        raise KernelError(f"expert_gate_up: shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    max_tiles = route_max_tiles(T * top, E)
+    _ints(tiles, 3 * max_tiles, "expert tiles"); _ints(n_tiles, 1, "tile count"); _ints(pair_of_row, T * top, "pair_of_row")
+    check(library().sp_expert_gate_up(_stream(), _code(w, "expert weights"), x.data_ptr(), w.data_ptr(), tiles.data_ptr(),
+                                      n_tiles.data_ptr(), max_tiles, pair_of_row.data_ptr(), top, out.data_ptr(), T, E,
+                                      two_i // 2, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+
+
+def expert_down(act: torch.Tensor, w: torch.Tensor, tiles, n_tiles, out: torch.Tensor) -> None:
+    """out[row] (float32) = act[row] . w[e]^T for every sorted row (w [experts, hidden, I])."""
+    _gpu(act, "expert activations"); _gpu(w, "expert down weights"); _gpu(out, "expert outputs")
+    rows, inner = act.shape
+    E, hidden, _ = w.shape
+    if w.shape[2] != inner or tuple(out.shape) != (rows, hidden) or out.dtype != torch.float32 or act.dtype != w.dtype:
+        raise KernelError(f"expert_down: shapes do not fit: act {tuple(act.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} {out.dtype}")
+    max_tiles = route_max_tiles(rows, E)
+    _ints(tiles, 3 * max_tiles, "expert tiles"); _ints(n_tiles, 1, "tile count")
+    check(library().sp_expert_down(_stream(), _code(w, "expert weights"), act.data_ptr(), w.data_ptr(), tiles.data_ptr(),
+                                   n_tiles.data_ptr(), max_tiles, out.data_ptr(), rows, E, hidden, inner))
+
+
+def route_combine(y: torch.Tensor, row_of_pair, weights: torch.Tensor, residual: torch.Tensor) -> None:
+    """residual[t] += sum_k weights[t, k] * y[row_of_pair[t * top + k]]."""
+    _gpu(y, "expert outputs"); _gpu(weights, "expert weights"); _gpu(residual, "residual")
+    T, top = weights.shape
+    H = residual.shape[1]
+    if y.dtype != torch.float32 or tuple(y.shape) != (T * top, H) or residual.dtype != torch.float32 or residual.shape[0] < T \
+            or weights.dtype != torch.float32:
+        raise KernelError("route_combine: float32 outputs [T * top, H], weights [T, top] and residual [T, H] expected")
+    _ints(row_of_pair, T * top, "row_of_pair")
+    check(library().sp_route_combine(_stream(), y.data_ptr(), row_of_pair.data_ptr(), weights.data_ptr(), top,
+                                     residual.data_ptr(), T, H))
 
 
 STORE, ACCUMULATE, STORE_F32 = 0, 1, 2

@@ -16,23 +16,26 @@ class GatedMLP(FeedForward):
 
     graph_safe_portions = True
 
-    def __init__(self, hidden: int, inner: int, activation: str = "silu"):
+    def __init__(self, hidden: int, inner: int, activation: str = "silu",
+                 tensors: tuple = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
         if activation not in ops.GATE_ACTIVATIONS:     # refused when the part is built, not at the first step
             raise ValueError(f"Gated feed-forward with activation {activation!r} has no kernel; "
                              f"there are kernels for {sorted(ops.GATE_ACTIVATIONS)}.")
         self.hidden, self.inner, self.activation = hidden, inner, activation
+        self.names = tuple(tensors)      # local names of the gate, up and down matrices
 
     def flops(self, tokens: int, pairs: int = 0) -> float:
         return 2.0 * tokens * 3 * self.hidden * self.inner
 
     def tensors(self):
-        return {"gate_proj.weight": TensorSpec((self.inner, self.hidden)),
-                "up_proj.weight": TensorSpec((self.inner, self.hidden)),
-                "down_proj.weight": TensorSpec((self.hidden, self.inner))}
+        gate, up, down = self.names
+        return {gate: TensorSpec((self.inner, self.hidden)), up: TensorSpec((self.inner, self.hidden)),
+                down: TensorSpec((self.hidden, self.inner))}
 
     def bind(self, tensors):
-        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
-        self.w_down = tensors["down_proj.weight"]
+        gate, up, down = self.names
+        self.w_gate_up = torch.cat([tensors[gate], tensors[up]], dim=0).contiguous()
+        self.w_down = tensors[down]
         self.w = {}
 
     def _fused(self, T: int, norm: bool) -> bool:

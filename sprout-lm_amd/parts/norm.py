@@ -1,4 +1,4 @@
-"""Learned RMSNorm (reference: norm, src/qwen.ts:72-77)."""
+"""Learned norms: RMSNorm (reference: norm, src/qwen.ts:72-77) and layer norm without bias."""
 from __future__ import annotations
 
 from .. import ops
@@ -26,3 +26,24 @@ class RMSNorm(Norm):
 
     def fold(self):
         return NormFold("rms", self.w["weight"], self.eps)
+
+
+@register_part("norm", "layernorm")
+class LayerNorm(Norm):
+    """y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight, no bias; sums in float32.  `tensor`: the local
+    name of the weight (checkpoints that call a norm's weight by the norm's own name give the name here and the
+    prefix up to it)."""
+
+    graph_safe = True
+
+    graph_safe_portions = True
+
+    def __init__(self, size: int, eps: float, tensor: str = "weight"):
+        self.size, self.eps, self.tensor = size, eps, tensor
+
+    def tensors(self):
+        return {self.tensor: TensorSpec((self.size,), "vector", "one_plus_normal")}
+
+    def forward(self, ctx, x, out, rows=None):
+        ops.layernorm(x, self.w[self.tensor], self.eps, out, rows)
+        return out

@@ -51,6 +51,53 @@ class NeoxRotary(PositionEncoding):
         return found
 
 
+@register_part("position", "rotary_interleaved")
+class InterleavedRotary(PositionEncoding):
+    """Neighbours (2i, 2i + 1) of the first `rotary_dim` numbers turn by position * f_i, f_i = theta^(-2i / rotary_dim).
+
+    `scaling` (None, or factor / original / fast / slow): frequencies are blended between f_i and f_i / factor
+    along a ramp over the pair index, and cosine and sine are multiplied by `magnitude` = 0.1 ln(factor) + 1
+    ("YaRN").  With turns(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(turns(fast)), 0),
+    hi = min(ceil(turns(slow)), rotary_dim - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) the
+    frequency of pair i is f_i / factor * ramp_i + f_i * (1 - ramp_i).
+
+    The table `freq` is float64 on the device; the kernels that turn (the latent mixer's) compute the angle in
+    float32 for bfloat16 models and in float64 for float32 models."""
+
+    graph_safe = True
+
+    graph_safe_portions = True
+    pairing = "interleaved"
+
+    def __init__(self, rotary_dim: int, theta: float, scaling: dict | None = None):
+        import math
+        if rotary_dim % 2 or rotary_dim < 0:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even.")
+        self.rotary_dim, self.theta, self.scaling = rotary_dim, float(theta), dict(scaling) if scaling else None
+        self.magnitude = 0.1 * math.log(float(self.scaling["factor"])) + 1.0 if self.scaling else 1.0
+        self.freq = None
+        self.inv_freq = None
+
+    def frequencies(self) -> torch.Tensor:
+        import math
+        n = self.rotary_dim
+        i = torch.arange(n // 2, dtype=torch.float64)
+        freq = self.theta ** (-2.0 * i / max(n, 1))
+        if not self.scaling:
+            return freq
+        factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+        turns = lambda t: n * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(self.theta))
+        lo = max(math.floor(turns(float(self.scaling["fast"]))), 0)
+        hi = min(math.ceil(turns(float(self.scaling["slow"]))), n - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        return freq / factor * ramp + freq * (1.0 - ramp)
+
+    def prepare(self, device, dtype):
+        exact = self.frequencies() if self.rotary_dim else torch.zeros(1, dtype=torch.float64)
+        self.freq = exact.to(device)
+        self.inv_freq = exact.to(torch.float32).to(device)
+
+
 @register_part("position", "none")
 class NoPosition(PositionEncoding):
     """No position encoding: queries and keys are used as projected."""

@@ -28,6 +28,11 @@ def resolve_architecture(raw: Mapping) -> str:
             if name in _ARCHITECTURES:
                 return name
         raise ConfigError(f"Unknown architecture {names!r}; registered: {registered_architectures()}.")
+    single = raw.get("architecture")       # some configurations name their one architecture under this key
+    if isinstance(single, str):
+        if single in _ARCHITECTURES:
+            return single
+        raise ConfigError(f"Unknown architecture {single!r}; registered: {registered_architectures()}.")
     model_type = raw.get("model_type")
     if model_type in _MODEL_TYPES:
         return _MODEL_TYPES[model_type]
@@ -57,6 +62,9 @@ def _register_builtin():
     from .config.qwen2 import Qwen2Config
     from .models.qwen2 import build_qwen2
     register_architecture(Qwen2Config.architecture, Qwen2Config, build_qwen2)
+    from .config.megozen import MegozenConfig
+    from .models.megozen import build_megozen
+    register_architecture(MegozenConfig.architecture, MegozenConfig, build_megozen)
 
 
 _register_builtin()
