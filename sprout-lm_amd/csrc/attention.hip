@@ -99,6 +99,11 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
                              ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages, window, scale,
                              max_tile_ctx, need ? workspace : nullptr, single);
   }
+  if (plan[1]) {      // groups too large for the one-query kernel: the tile list holds every sequence, and that a step
+    n_decode = 0;     // brings one query a sequence (n_decode == n_tiles) is a hint this kernel has no use for
+    decode_seqs = nullptr;
+    max_decode_ctx = 0;
+  }
   SP_REQUIRE(max_decode_ctx >= 0 && max_decode_ctx <= max_blocks * page_size,
              "sp_attention: decode context %d exceeds the block tables", max_decode_ctx);
   SP_REQUIRE(max_tile_ctx >= 0, "sp_attention: negative context length");

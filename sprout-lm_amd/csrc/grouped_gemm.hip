@@ -5,34 +5,13 @@
 //
 // This file holds the float32-arithmetic form (FMA, any sizes and both storage types): tiles of 64 rows x 64
 // columns, steps of 16 along K through LDS, a thread a 4 x 4 patch.
-#include "common.h"
+#include "grouped_gemm.h"
 #include "sprout_hip.h"
 
 namespace sprout {
 
 constexpr int GT = 64;     // rows and columns of a tile
 constexpr int GK = 16;     // step along K
-
-struct GroupedArgs {
-  const void* a;            // operand rows
-  long long a_stride;       // between rows
-  long long a_group_stride; // between the groups' column ranges of a row (0: every group reads the same columns)
-  const int32_t* gather;    // row r of the list reads operand row gather[r] / gather_div (null: row r)
-  int gather_div;
-  const void* w;            // [groups][rows of K]
-  long long w_group_stride;
-  void* out;
-  long long out_stride, out_group_stride;
-  const void* gate;         // epilogue 2: out *= sigmoid(gate[row * gate_stride + group])
-  long long gate_stride;
-  const int32_t* tiles;     // [n][3] = group, first row, rows (null: every group owns `rows`, in tiles_per_group tiles)
-  const int32_t* n_tiles;
-  int rows, tiles_per_group;
-  int N, K;
-  int up_offset;            // epilogue 1: weight row n is the gate's, row up_offset + n the matching up row
-};
-
-enum { kStore = 0, kGated = 1, kSigmoid = 2 };
 
 template <typename TA, typename TO, int MODE>
 __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs p) {
@@ -130,7 +109,21 @@ static int launch_grouped(hipStream_t s, int dtype, int out_dtype, const Grouped
 
 using namespace sprout;
 
-extern "C" int sp_group_tile_rows() { return GT; }
+// Rows a tile of the grouped products holds: 128 where a group brings at least that many rows and the matrix-core
+// kernels take the sizes (bfloat16, K in eights), else 64.
+extern "C" int sp_group_tile_rows(int dtype, long long rows, int groups, int K) {
+  return (dtype == kBF16 && K % 8 == 0 && groups > 0 && rows / groups >= 128) ? 128 : GT;
+}
+
+// The float32-arithmetic kernel cuts its own tiles of 64 rows; a list cut for more rows is not for it.
+static int grouped(hipStream_t s, int mode, int dtype, int out_dtype, const GroupedArgs& p, int tiles, int tile_rows,
+                   const char* what) {
+  if (grouped_mfma_takes(dtype, p)) return launch_grouped_mfma(s, mode, out_dtype, p, tiles, tile_rows, what);
+  SP_REQUIRE(tile_rows == GT, "%s: tiles of %d rows need operands the matrix-core kernels take", what, tile_rows);
+  if (mode == kGated) return launch_grouped<kGated>(s, dtype, out_dtype, p, tiles, what);
+  if (mode == kSigmoid) return launch_grouped<kSigmoid>(s, dtype, out_dtype, p, tiles, what);
+  return launch_grouped<kStore>(s, dtype, out_dtype, p, tiles, what);
+}
 
 extern "C" int sp_head_gemm(void* stream, int dtype, const void* a, long long a_stride, long long a_head_stride,
                             const void* w, void* out, long long out_stride, long long out_head_stride, const void* gate,
@@ -145,18 +138,18 @@ extern "C" int sp_head_gemm(void* stream, int dtype, const void* a, long long a_
   p.w = w; p.w_group_stride = (long long)N * K;
   p.out = out; p.out_stride = out_stride; p.out_group_stride = out_head_stride;
   p.gate = gate; p.gate_stride = gate_stride;
-  p.rows = T; p.tiles_per_group = (T + GT - 1) / GT;
+  p.rows = T;
   p.N = N; p.K = K;
+  const int tile_rows = (grouped_mfma_takes(dtype, p) && T >= 256) ? 128 : GT;
+  p.tiles_per_group = (T + tile_rows - 1) / tile_rows;
   const long long blocks = (long long)heads * p.tiles_per_group;
   SP_REQUIRE(blocks < (1ll << 31), "sp_head_gemm: too many tiles");
-  hipStream_t s = (hipStream_t)stream;
-  return gate ? launch_grouped<kSigmoid>(s, dtype, dtype, p, int(blocks), "sp_head_gemm")
-              : launch_grouped<kStore>(s, dtype, dtype, p, int(blocks), "sp_head_gemm");
+  return grouped((hipStream_t)stream, gate ? kSigmoid : kStore, dtype, dtype, p, int(blocks), tile_rows, "sp_head_gemm");
 }
 
 extern "C" int sp_expert_gate_up(void* stream, int dtype, const void* x, const void* w, const int32_t* tiles,
-                                 const int32_t* n_tiles, int max_tiles, const int32_t* pair_of_row, int top, void* out,
-                                 int T, int experts, int inner, int K, int activation) {
+                                 const int32_t* n_tiles, int max_tiles, int tile_rows, const int32_t* pair_of_row, int top,
+                                 void* out, int T, int experts, int inner, int K, int activation) {
   SP_REQUIRE(activation == 0, "sp_expert_gate_up: no kernel for activation %d (0 = SiLU)", activation);
   SP_REQUIRE(T >= 0 && experts > 0 && inner > 0 && K > 0 && top > 0 && max_tiles > 0, "sp_expert_gate_up: bad sizes");
   SP_REQUIRE(x && w && tiles && n_tiles && pair_of_row && out, "sp_expert_gate_up: null operand");
@@ -167,12 +160,12 @@ extern "C" int sp_expert_gate_up(void* stream, int dtype, const void* x, const v
   p.out = out; p.out_stride = inner;
   p.tiles = tiles; p.n_tiles = n_tiles;
   p.N = inner; p.K = K; p.up_offset = inner;
-  return launch_grouped<kGated>((hipStream_t)stream, dtype, dtype, p, max_tiles, "sp_expert_gate_up");
+  return grouped((hipStream_t)stream, kGated, dtype, dtype, p, max_tiles, tile_rows, "sp_expert_gate_up");
 }
 
 extern "C" int sp_expert_down(void* stream, int dtype, const void* act, const void* w, const int32_t* tiles,
-                              const int32_t* n_tiles, int max_tiles, float* out, int rows, int experts, int hidden,
-                              int inner) {
+                              const int32_t* n_tiles, int max_tiles, int tile_rows, float* out, int rows, int experts,
+                              int hidden, int inner) {
   SP_REQUIRE(rows >= 0 && experts > 0 && inner > 0 && hidden > 0 && max_tiles > 0, "sp_expert_down: bad sizes");
   SP_REQUIRE(act && w && tiles && n_tiles && out, "sp_expert_down: null operand");
   if (rows == 0) return 0;
@@ -182,5 +175,5 @@ extern "C" int sp_expert_down(void* stream, int dtype, const void* act, const vo
   p.out = out; p.out_stride = hidden;
   p.tiles = tiles; p.n_tiles = n_tiles;
   p.N = hidden; p.K = inner;
-  return launch_grouped<kStore>((hipStream_t)stream, dtype, kF32, p, max_tiles, "sp_expert_down");
+  return grouped((hipStream_t)stream, kStore, dtype, kF32, p, max_tiles, tile_rows, "sp_expert_down");
 }

@@ -1,0 +1,168 @@
+// Grouped products on the matrix cores (bfloat16 operands, float32 sums): the per-head products of attention over
+// a latent and the experts of a routed feed-forward, see grouped_gemm.hip for what a group is.
+//
+// A block of four waves owns a tile of BM rows x BN columns (64 or 128 each) of one group and walks K in steps of
+// 64: the rows of a (gathered through the pair list where there is one) and the rows of w go from memory to
+// registers to LDS in 16-byte pieces, the next step's pieces asked for before the current step is multiplied.  A
+// wave owns a quarter of the tile, as 32x32x16 MFMA tiles.  Rows behind a tile's last row and columns behind N
+// are zeros in LDS and are not stored.  Epilogues: store; SiLU(gate) * up with the up rows in a second set of
+// accumulators; multiplication by sigmoid of a per-(row, group) gate.
+#include "grouped_gemm.h"
+#include "mfma.h"
+#include "sprout_hip.h"
+
+namespace sprout {
+
+constexpr int GBK = 64;          // step along K
+constexpr int GLD = GBK + 8;     // bf16 numbers a row of LDS (16 bytes of padding: neighbouring rows start 4 banks apart)
+
+template <int BM, int BN, int MODE, typename TO>
+__global__ __launch_bounds__(256) void grouped_mfma_kernel(GroupedArgs p) {
+  constexpr int TM = BM / 64, TN = BN / 64;       // 32x32 tiles of a wave along rows and columns
+  constexpr int A_CH = BM / 32, W_CH = BN / 32;   // 16-byte pieces a thread moves per step: rows tid / 8 + 32 j, piece tid % 8
+  constexpr bool GATED = MODE == kGated;
+  __shared__ __attribute__((aligned(16))) uint16_t As[BM * GLD];
+  __shared__ __attribute__((aligned(16))) uint16_t Ws[BN * GLD];
+  __shared__ __attribute__((aligned(16))) uint16_t Us[GATED ? BN * GLD : 8];
+  int group, row0, nrows;
+  if (p.tiles) {
+    if (int(blockIdx.x) >= *p.n_tiles) return;
+    group = p.tiles[3 * blockIdx.x];
+    row0 = p.tiles[3 * blockIdx.x + 1];
+    nrows = p.tiles[3 * blockIdx.x + 2];
+  } else {
+    group = blockIdx.x / p.tiles_per_group;
+    row0 = (blockIdx.x - group * p.tiles_per_group) * BM;
+    nrows = min(BM, p.rows - row0);
+  }
+  const int n0 = blockIdx.y * BN;
+  const int tid = threadIdx.x, piece = tid & 7, lrow = tid >> 3;
+  const uint16_t* a_ptr[A_CH];
+  const uint16_t* w_ptr[W_CH];
+  const uint16_t* u_ptr[W_CH];
+#pragma unroll
+  for (int j = 0; j < A_CH; ++j) {
+    const int r = lrow + 32 * j;
+    a_ptr[j] = nullptr;
+    if (r < nrows) {
+      const long long src = p.gather ? p.gather[row0 + r] / p.gather_div : row0 + r;
+      a_ptr[j] = (const uint16_t*)p.a + src * p.a_stride + group * p.a_group_stride + 8 * piece;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < W_CH; ++j) {
+    const int n = n0 + lrow + 32 * j;
+    const uint16_t* base = (const uint16_t*)p.w + group * p.w_group_stride + 8 * piece;
+    w_ptr[j] = n < p.N ? base + (long long)n * p.K : nullptr;
+    u_ptr[j] = (GATED && n < p.N) ? base + (long long)(p.up_offset + n) * p.K : nullptr;
+  }
+  uint4 a_reg[A_CH], w_reg[W_CH], u_reg[GATED ? W_CH : 1];
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  auto fetch = [&](int k0) {
+    const bool in_k = k0 + 8 * piece < p.K;      // K is a multiple of 8: a piece is inside or outside as a whole
+#pragma unroll
+    for (int j = 0; j < A_CH; ++j) a_reg[j] = (a_ptr[j] && in_k) ? ldg128(a_ptr[j] + k0) : zero;
+#pragma unroll
+    for (int j = 0; j < W_CH; ++j) {
+      w_reg[j] = (w_ptr[j] && in_k) ? ldg128(w_ptr[j] + k0) : zero;
+      if (GATED) u_reg[j] = (u_ptr[j] && in_k) ? ldg128(u_ptr[j] + k0) : zero;
+    }
+  };
+  const int wave = tid >> 6, lane = tid & 63, lr = lane & 31, lk = lane >> 5;
+  const int wm = (wave >> 1) * (BM / 2), wn = (wave & 1) * (BN / 2);
+  floatx16 acc[TM][TN], acc2[GATED ? TM : 1][GATED ? TN : 1];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      if (GATED) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc2[i][j][r] = 0.f;
+      }
+    }
+  fetch(0);
+  for (int k0 = 0; k0 < p.K; k0 += GBK) {
+#pragma unroll
+    for (int j = 0; j < A_CH; ++j) *reinterpret_cast<uint4*>(&As[(lrow + 32 * j) * GLD + 8 * piece]) = a_reg[j];
+#pragma unroll
+    for (int j = 0; j < W_CH; ++j) {
+      *reinterpret_cast<uint4*>(&Ws[(lrow + 32 * j) * GLD + 8 * piece]) = w_reg[j];
+      if (GATED) *reinterpret_cast<uint4*>(&Us[(lrow + 32 * j) * GLD + 8 * piece]) = u_reg[j];
+    }
+    __syncthreads();
+    if (k0 + GBK < p.K) fetch(k0 + GBK);
+#pragma unroll
+    for (int kk = 0; kk < GBK / 16; ++kk) {
+      bf16x8 av[TM], wv[TN], uv[GATED ? TN : 1];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        av[i] = as_bf16x8(*reinterpret_cast<const uint4*>(&As[(wm + 32 * i + lr) * GLD + 16 * kk + 8 * lk]));
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        wv[j] = as_bf16x8(*reinterpret_cast<const uint4*>(&Ws[(wn + 32 * j + lr) * GLD + 16 * kk + 8 * lk]));
+        if (GATED) uv[j] = as_bf16x8(*reinterpret_cast<const uint4*>(&Us[(wn + 32 * j + lr) * GLD + 16 * kk + 8 * lk]));
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          acc[i][j] = mfma32(av[i], wv[j], acc[i][j]);
+          if (GATED) acc2[i][j] = mfma32(av[i], uv[j], acc2[i][j]);
+        }
+    }
+    __syncthreads();
+  }
+  // lane l, number r of a 32x32 tile: row 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = wm + 32 * i + 8 * (r >> 2) + 4 * lk + (r & 3);
+      if (row >= nrows) continue;
+      float g = 1.f;
+      if (MODE == kSigmoid)
+        g = 1.0f / (1.0f + expf(-to_float(((const bf16_t*)p.gate)[(long long)(row0 + row) * p.gate_stride + group])));
+      TO* o = (TO*)p.out + (long long)(row0 + row) * p.out_stride + group * p.out_group_stride;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn + 32 * j + lr;
+        if (n >= p.N) continue;
+        float v = acc[i][j][r];
+        if (GATED) v = (v / (1.0f + expf(-v))) * acc2[i][j][r];
+        if (MODE == kSigmoid) v *= g;
+        o[n] = from_float<TO>(v);
+      }
+    }
+}
+
+bool grouped_mfma_takes(int dtype, const GroupedArgs& p) {
+  auto whole = [](long long n) { return n % 8 == 0; };
+  return dtype == kBF16 && p.K > 0 && whole(p.K) && whole(p.a_stride) && whole(p.a_group_stride) && whole(p.w_group_stride) &&
+         whole((long long)p.up_offset * p.K) && (uintptr_t)p.a % 16 == 0 && (uintptr_t)p.w % 16 == 0;
+}
+
+template <int BM, int BN>
+static int launch_shape(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, const char* what) {
+  dim3 grid(tiles, (p.N + BN - 1) / BN);
+  if (mode == kStore && out_dtype == kBF16) grouped_mfma_kernel<BM, BN, kStore, bf16_t><<<grid, 256, 0, s>>>(p);
+  else if (mode == kStore && out_dtype == kF32) grouped_mfma_kernel<BM, BN, kStore, float><<<grid, 256, 0, s>>>(p);
+  else if (mode == kGated && out_dtype == kBF16) grouped_mfma_kernel<BM, BN, kGated, bf16_t><<<grid, 256, 0, s>>>(p);
+  else if (mode == kSigmoid && out_dtype == kBF16) grouped_mfma_kernel<BM, BN, kSigmoid, bf16_t><<<grid, 256, 0, s>>>(p);
+  else SP_REQUIRE(false, "%s: no matrix-core kernel for epilogue %d with output type %d", what, mode, out_dtype);
+  return check_launch(what);
+}
+
+int launch_grouped_mfma(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, int tile_rows,
+                        const char* what) {
+  SP_REQUIRE(tile_rows == 64 || tile_rows == 128, "%s: tiles of %d rows", what, tile_rows);
+  // wide tiles where there are columns for them; the gated epilogue keeps two sets of accumulators
+  const bool wide = p.N > 64;
+  if (tile_rows == 128) return wide ? launch_shape<128, 128>(s, mode, out_dtype, p, tiles, what)
+                                    : launch_shape<128, 64>(s, mode, out_dtype, p, tiles, what);
+  return wide ? launch_shape<64, 128>(s, mode, out_dtype, p, tiles, what)
+              : launch_shape<64, 64>(s, mode, out_dtype, p, tiles, what);
+}
+
+}  // namespace sprout

@@ -7,9 +7,11 @@ namespace sprout {
 
 // y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w.  One block a row; the row is read three times (the second
 // and third time from the caches): the variance is the mean of the squared deviations, not E[x^2] - mean^2.
+// With w2 and out2 the same normalised row is also written times a second weight (two norms of one input).
 template <typename TW, typename TO>
 __global__ void layernorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
-                                 const TW* __restrict__ w, float eps, TO* __restrict__ out, int H) {
+                                 const TW* __restrict__ w, const TW* __restrict__ w2, float eps, TO* __restrict__ out,
+                                 TO* __restrict__ out2, int H) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const float* in = x + size_t(rows ? rows[r] : r) * H;
@@ -23,7 +25,12 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int32_t* __r
   }
   const float scale = 1.0f / sqrtf(block_sum(sq, scratch) / float(H) + eps);
   TO* o = out + size_t(r) * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<TO>(((in[i] - mean) * scale) * to_float(w[i]));
+  TO* o2 = out2 ? out2 + size_t(r) * H : nullptr;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    const float y = (in[i] - mean) * scale;
+    o[i] = from_float<TO>(y * to_float(w[i]));
+    if (o2) o2[i] = from_float<TO>(y * to_float(w2[i]));
+  }
 }
 
 // residual[t] = table[token] + pairs[row], row = (previous * mul_prev + token * mul_cur) mod buckets, and row
@@ -66,22 +73,21 @@ __global__ void embed_bigram_kernel(const TW* __restrict__ table, const TW* __re
 
 using namespace sprout;
 
-extern "C" int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, float eps,
-                            int out_dtype, void* out, int R, int H) {
+extern "C" int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, const void* w2,
+                            float eps, int out_dtype, void* out, void* out2, int R, int H) {
   SP_REQUIRE(R >= 0 && H > 0 && x && w && out, "sp_layernorm: bad arguments R=%d H=%d", R, H);
+  SP_REQUIRE((w2 == nullptr) == (out2 == nullptr), "sp_layernorm: a second weight goes with a second output");
   if (R == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int threads = H >= 2048 ? 512 : 256;
-  if (w_dtype == kF32 && out_dtype == kF32)
-    layernorm_kernel<float, float><<<R, threads, 0, s>>>(x, rows, (const float*)w, eps, (float*)out, H);
-  else if (w_dtype == kF32 && out_dtype == kBF16)
-    layernorm_kernel<float, bf16_t><<<R, threads, 0, s>>>(x, rows, (const float*)w, eps, (bf16_t*)out, H);
-  else if (w_dtype == kBF16 && out_dtype == kF32)
-    layernorm_kernel<bf16_t, float><<<R, threads, 0, s>>>(x, rows, (const bf16_t*)w, eps, (float*)out, H);
-  else if (w_dtype == kBF16 && out_dtype == kBF16)
-    layernorm_kernel<bf16_t, bf16_t><<<R, threads, 0, s>>>(x, rows, (const bf16_t*)w, eps, (bf16_t*)out, H);
-  else
-    SP_REQUIRE(false, "sp_layernorm: unsupported dtypes w=%d out=%d", w_dtype, out_dtype);
+#define SP_LN(TW, TO) \
+  layernorm_kernel<TW, TO><<<R, threads, 0, s>>>(x, rows, (const TW*)w, (const TW*)w2, eps, (TO*)out, (TO*)out2, H)
+  if (w_dtype == kF32 && out_dtype == kF32) SP_LN(float, float);
+  else if (w_dtype == kF32 && out_dtype == kBF16) SP_LN(float, bf16_t);
+  else if (w_dtype == kBF16 && out_dtype == kF32) SP_LN(bf16_t, float);
+  else if (w_dtype == kBF16 && out_dtype == kBF16) SP_LN(bf16_t, bf16_t);
+  else SP_REQUIRE(false, "sp_layernorm: unsupported dtypes w=%d out=%d", w_dtype, out_dtype);
+#undef SP_LN
   return check_launch("sp_layernorm");
 }
 

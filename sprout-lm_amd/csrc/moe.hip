@@ -6,15 +6,10 @@
 
 namespace sprout {
 
-// One thread a token: the `top` largest of its `experts` logits (the lowest index wins a tie), in falling order,
-// and the softmax over the chosen logits alone.
-__global__ void route_topk_kernel(const float* __restrict__ logits, int experts, int top, int32_t* __restrict__ ids,
-                                  float* __restrict__ weights, int T) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= T) return;
-  const float* z = logits + size_t(t) * experts;
-  int32_t* id = ids + size_t(t) * top;
-  float* w = weights + size_t(t) * top;
+// The `top` largest of a token's `experts` logits (the lowest index wins a tie), in falling order, and the softmax
+// over the chosen logits alone.
+__device__ __forceinline__ void route_token(const float* __restrict__ z, int experts, int top, int32_t* __restrict__ id,
+                                            float* __restrict__ w) {
   for (int k = 0; k < top; ++k) {
     int best = -1;
     float best_z = 0.f;
@@ -33,15 +28,29 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, int experts,
   for (int k = 0; k < top; ++k) w[k] /= sum;
 }
 
+// One thread a token.
+__global__ void route_topk_kernel(const float* __restrict__ logits, int experts, int top, int32_t* __restrict__ ids,
+                                  float* __restrict__ weights, int T) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  route_token(logits + size_t(t) * experts, experts, top, ids + size_t(t) * top, weights + size_t(t) * top);
+}
+
 // One block: sorts the pairs (token, choice) by expert.  row_of_pair[p] = the row of pair p in the sorted order,
 // pair_of_row its inverse; tiles [n][3] = (expert, first row, rows) cuts every expert's rows into tiles of at most
 // tile_rows; *n_tiles = n.  Within an expert the rows stand in no fixed order (every row is computed for itself).
-__global__ void route_sort_kernel(const int32_t* __restrict__ ids, int pairs, int experts, int tile_rows,
+// With `logits` (and `weights`, `top`) the block first makes the choice itself (ids and weights are then outputs):
+// choice and order in one launch.
+__global__ void route_sort_kernel(const float* __restrict__ logits, float* __restrict__ weights, int top,
+                                  int32_t* __restrict__ ids, int pairs, int experts, int tile_rows,
                                   int32_t* __restrict__ row_of_pair, int32_t* __restrict__ pair_of_row,
                                   int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles) {
   extern __shared__ int32_t count[];      // [experts] counts, then [experts] first rows
   int32_t* first = count + experts;
   for (int e = threadIdx.x; e < experts; e += blockDim.x) count[e] = 0;
+  if (logits)
+    for (int t = threadIdx.x; t < pairs / top; t += blockDim.x)
+      route_token(logits + size_t(t) * experts, experts, top, ids + size_t(t) * top, weights + size_t(t) * top);
   __syncthreads();
   for (int p = threadIdx.x; p < pairs; p += blockDim.x) row_of_pair[p] = atomicAdd(&count[ids[p]], 1);
   __syncthreads();
@@ -101,8 +110,26 @@ extern "C" int sp_route_sort(void* stream, const int32_t* ids, int pairs, int ex
   SP_REQUIRE(pairs >= 0 && experts > 0 && experts <= 8192 && tile_rows > 0, "sp_route_sort: bad sizes");
   SP_REQUIRE(ids && row_of_pair && pair_of_row && tiles && n_tiles, "sp_route_sort: null operand");
   route_sort_kernel<<<1, 1024, 2 * size_t(experts) * sizeof(int32_t), (hipStream_t)stream>>>(
-      ids, pairs, experts, tile_rows, row_of_pair, pair_of_row, tiles, n_tiles);
+      nullptr, nullptr, 1, const_cast<int32_t*>(ids), pairs, experts, tile_rows, row_of_pair, pair_of_row, tiles, n_tiles);
   return check_launch("sp_route_sort");
+}
+
+extern "C" int sp_route(void* stream, const float* logits, int32_t* ids, float* weights, int T, int experts, int top,
+                        int tile_rows, int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles) {
+  SP_REQUIRE(T >= 0 && experts > 0 && experts <= 8192 && top > 0 && top <= experts && tile_rows > 0, "sp_route: bad sizes");
+  SP_REQUIRE(logits && ids && weights && row_of_pair && pair_of_row && tiles && n_tiles, "sp_route: null operand");
+  hipStream_t s = (hipStream_t)stream;
+  const size_t lds = 2 * size_t(experts) * sizeof(int32_t);
+  if (T <= 8192) {      // one block does both: a launch less in the chain of a step
+    route_sort_kernel<<<1, 1024, lds, s>>>(logits, weights, top, ids, T * top, experts, tile_rows, row_of_pair, pair_of_row,
+                                           tiles, n_tiles);
+    return check_launch("sp_route");
+  }
+  route_topk_kernel<<<(T + 63) / 64, 64, 0, s>>>(logits, experts, top, ids, weights, T);
+  if (check_launch("sp_route (choice)")) return 1;
+  route_sort_kernel<<<1, 1024, lds, s>>>(nullptr, nullptr, 1, ids, T * top, experts, tile_rows, row_of_pair, pair_of_row,
+                                         tiles, n_tiles);
+  return check_launch("sp_route (order)");
 }
 
 extern "C" int sp_route_combine(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,

@@ -156,9 +156,9 @@ int sp_sample_static(void* stream, const float* logits, const float* temperature
 int sp_sample_static_max_floats();
 
 // Layer norm without bias: out[r, :] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w, x float32 [*, H], rows as in
-// sp_rmsnorm.
-int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, float eps,
-                 int out_dtype, void* out, int R, int H);
+// sp_rmsnorm.  With w2 and out2 (both or neither) the normalised row is also written times a second weight.
+int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, const void* w2, float eps,
+                 int out_dtype, void* out, void* out2, int R, int H);
 
 // residual[t, :] = table[tokens[t], :] + pairs[row, :] with row = (previous * mul_prev + tokens[t] * mul_cur) mod buckets,
 // and row `buckets` (the table's last) at position 0.  The token before a step's first token of a sequence is read
@@ -196,17 +196,22 @@ int sp_head_gemm(void* stream, int dtype, const void* a, long long a_stride, lon
 // out[row, :] = act(x[token] . w[e][:inner]^T) * (x[token] . w[e][inner:]^T) for the rows of every tile (token =
 // pair_of_row[row] / top; w [experts, 2 inner, K]).  sp_expert_down: out[row, :] = act[row] . w[e]^T in float32
 // (w [experts, hidden, inner]).  sp_route_combine: residual[t] += sum_k weights[t, k] * y[row_of_pair[t * top + k]].
-// sp_group_tile_rows(): the tile_rows that the grouped products take.
-int sp_group_tile_rows();
+// sp_group_tile_rows: the tile_rows to cut the list for: 128 where the `groups` own `rows` rows of which a group has
+// at least 128 on average and the matrix-core kernels take the operands (`dtype` bfloat16, K in eights), else 64.
+// The float32-arithmetic kernel takes lists cut for 64 only.
+int sp_group_tile_rows(int dtype, long long rows, int groups, int K);
 int sp_route_topk(void* stream, const float* logits, int32_t* ids, float* weights, int T, int experts, int top);
 int sp_route_max_tiles(int pairs, int experts, int tile_rows);
 int sp_route_sort(void* stream, const int32_t* ids, int pairs, int experts, int tile_rows, int32_t* row_of_pair,
                   int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
 int sp_expert_gate_up(void* stream, int dtype, const void* x, const void* w, const int32_t* tiles, const int32_t* n_tiles,
-                      int max_tiles, const int32_t* pair_of_row, int top, void* out, int T, int experts, int inner, int K,
-                      int activation);
+                      int max_tiles, int tile_rows, const int32_t* pair_of_row, int top, void* out, int T, int experts,
+                      int inner, int K, int activation);
 int sp_expert_down(void* stream, int dtype, const void* act, const void* w, const int32_t* tiles, const int32_t* n_tiles,
-                   int max_tiles, float* out, int rows, int experts, int hidden, int inner);
+                   int max_tiles, int tile_rows, float* out, int rows, int experts, int hidden, int inner);
+// sp_route: sp_route_topk and sp_route_sort in one call (one launch up to 8,192 tokens).
+int sp_route(void* stream, const float* logits, int32_t* ids, float* weights, int T, int experts, int top, int tile_rows,
+             int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
 int sp_route_combine(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,
                      float* residual, int T, int H);
 

@@ -122,18 +122,26 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
                                float(eps), _code(out, "norm output"), out.data_ptr(), R, H))
 
 
-def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
-    """out[r] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight of x[rows[r]] or x[r]; x is float32."""
+def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None,
+              weight2: torch.Tensor | None = None, out2: torch.Tensor | None = None) -> None:
+    """out[r] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight of x[rows[r]] or x[r]; x is float32.  With weight2
+    and out2 the same normalised row times a second weight goes to out2 (two norms of one input in one pass)."""
     _gpu(x, "norm input"); _gpu(weight, "norm weight"); _gpu(out, "norm output")
     R, H = out.shape
     if x.dtype != torch.float32 or x.shape[1] != H or weight.numel() != H:
         raise KernelError(f"layernorm: shapes do not fit: x {tuple(x.shape)} {x.dtype}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
+    if (weight2 is None) != (out2 is None):
+        raise KernelError("layernorm: a second weight goes with a second output")
+    if weight2 is not None:
+        _gpu(weight2, "second norm weight"); _gpu(out2, "second norm output")
+        if weight2.dtype != weight.dtype or weight2.numel() != H or out2.dtype != out.dtype or tuple(out2.shape) != (R, H):
+            raise KernelError("layernorm: the second weight and output must be shaped and typed like the first")
     if rows is not None:
         _ints(rows, R, "norm rows")
     elif x.shape[0] < R:
         raise KernelError("layernorm: fewer input rows than output rows")
     check(library().sp_layernorm(_stream(), x.data_ptr(), _ptr(rows), _code(weight, "norm weight"), weight.data_ptr(),
-                                 float(eps), _code(out, "norm output"), out.data_ptr(), R, H))
+                                 _ptr(weight2), float(eps), _code(out, "norm output"), out.data_ptr(), _ptr(out2), R, H))
 
 
 def embed_bigram(table: torch.Tensor, pairs: torch.Tensor, tokens, positions, q_start, q_len, seq_of_token, state_slots,
@@ -208,12 +216,14 @@ def head_gemm(a: torch.Tensor, a_offset: int, a_head_stride: int, w: torch.Tenso
                                  out_head_stride, gate_ptr, gate_stride, T, heads, N, K))
 
 
-def group_tile_rows() -> int:
-    return library().sp_group_tile_rows()
+def group_tile_rows(dtype: torch.dtype = torch.float32, rows: int = 0, groups: int = 1, eights: bool = False) -> int:
+    """Rows a tile of the grouped products holds: 128 where the groups own at least that many rows each on average and
+    the matrix-core kernels take the operands (bfloat16, every K in `eights`), else 64."""
+    return library().sp_group_tile_rows(_CODES[dtype], int(rows), int(groups), 8 if eights else 1)
 
 
-def route_max_tiles(pairs: int, experts: int) -> int:
-    return library().sp_route_max_tiles(pairs, experts, group_tile_rows())
+def route_max_tiles(pairs: int, experts: int, tile_rows: int = 64) -> int:
+    return library().sp_route_max_tiles(pairs, experts, tile_rows)
 
 
 def route_topk(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> None:
@@ -228,41 +238,57 @@ def route_topk(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -
     check(library().sp_route_topk(_stream(), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E, top))
 
 
-def route_sort(ids: torch.Tensor, experts: int, row_of_pair, pair_of_row, tiles, n_tiles) -> None:
+def route(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, row_of_pair, pair_of_row, tiles, n_tiles,
+          tile_rows: int = 64) -> None:
+    """route_topk and route_sort in one call (one launch for steps of up to 8,192 tokens)."""
+    _gpu(logits, "router logits"); _gpu(ids, "chosen experts"); _gpu(weights, "expert weights")
+    T, E = logits.shape
+    top = ids.shape[1]
+    if logits.dtype != torch.float32 or ids.dtype != torch.int32 or weights.dtype != torch.float32 or \
+            tuple(ids.shape) != (T, top) or tuple(weights.shape) != (T, top) or not 0 < top <= E:
+        raise KernelError("route: float32 logits [T, E], int32 ids and float32 weights [T, top] expected")
+    pairs = T * top
+    _ints(row_of_pair, pairs, "row_of_pair"); _ints(pair_of_row, pairs, "pair_of_row")
+    _ints(tiles, 3 * route_max_tiles(pairs, E, tile_rows), "expert tiles"); _ints(n_tiles, 1, "tile count")
+    check(library().sp_route(_stream(), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E, top, tile_rows,
+                             row_of_pair.data_ptr(), pair_of_row.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr()))
+
+
+def route_sort(ids: torch.Tensor, experts: int, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows: int = 64) -> None:
     """Orders the (token, choice) pairs by expert for the grouped products (see sprout_hip.h)."""
     pairs = ids.numel()
     _ints(ids, pairs, "chosen experts"); _ints(row_of_pair, pairs, "row_of_pair"); _ints(pair_of_row, pairs, "pair_of_row")
-    _ints(tiles, 3 * route_max_tiles(pairs, experts), "expert tiles"); _ints(n_tiles, 1, "tile count")
-    check(library().sp_route_sort(_stream(), ids.data_ptr(), pairs, experts, group_tile_rows(), row_of_pair.data_ptr(),
+    _ints(tiles, 3 * route_max_tiles(pairs, experts, tile_rows), "expert tiles"); _ints(n_tiles, 1, "tile count")
+    check(library().sp_route_sort(_stream(), ids.data_ptr(), pairs, experts, tile_rows, row_of_pair.data_ptr(),
                                   pair_of_row.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr()))
 
 
 def expert_gate_up(x: torch.Tensor, w: torch.Tensor, tiles, n_tiles, pair_of_row, top: int, out: torch.Tensor,
-                   activation: str = "silu") -> None:
+                   activation: str = "silu", tile_rows: int = 64) -> None:
     """out[row] = act(x[token] . w[e, :I]^T) * (x[token] . w[e, I:]^T) for every sorted row (w [experts, 2 I, K])."""
     _gpu(x, "expert input"); _gpu(w, "expert gate/up weights"); _gpu(out, "expert activations")
     T, K = x.shape
     E, two_i, _ = w.shape
     if w.shape[2] != K or two_i % 2 or tuple(out.shape) != (T * top, two_i // 2) or not (x.dtype == w.dtype == out.dtype):
         raise KernelError(f"expert_gate_up: shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
-    max_tiles = route_max_tiles(T * top, E)
+    max_tiles = route_max_tiles(T * top, E, tile_rows)
     _ints(tiles, 3 * max_tiles, "expert tiles"); _ints(n_tiles, 1, "tile count"); _ints(pair_of_row, T * top, "pair_of_row")
     check(library().sp_expert_gate_up(_stream(), _code(w, "expert weights"), x.data_ptr(), w.data_ptr(), tiles.data_ptr(),
-                                      n_tiles.data_ptr(), max_tiles, pair_of_row.data_ptr(), top, out.data_ptr(), T, E,
-                                      two_i // 2, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+                                      n_tiles.data_ptr(), max_tiles, tile_rows, pair_of_row.data_ptr(), top, out.data_ptr(),
+                                      T, E, two_i // 2, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
 
 
-def expert_down(act: torch.Tensor, w: torch.Tensor, tiles, n_tiles, out: torch.Tensor) -> None:
+def expert_down(act: torch.Tensor, w: torch.Tensor, tiles, n_tiles, out: torch.Tensor, tile_rows: int = 64) -> None:
     """out[row] (float32) = act[row] . w[e]^T for every sorted row (w [experts, hidden, I])."""
     _gpu(act, "expert activations"); _gpu(w, "expert down weights"); _gpu(out, "expert outputs")
     rows, inner = act.shape
     E, hidden, _ = w.shape
     if w.shape[2] != inner or tuple(out.shape) != (rows, hidden) or out.dtype != torch.float32 or act.dtype != w.dtype:
         raise KernelError(f"expert_down: shapes do not fit: act {tuple(act.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} {out.dtype}")
-    max_tiles = route_max_tiles(rows, E)
+    max_tiles = route_max_tiles(rows, E, tile_rows)
     _ints(tiles, 3 * max_tiles, "expert tiles"); _ints(n_tiles, 1, "tile count")
     check(library().sp_expert_down(_stream(), _code(w, "expert weights"), act.data_ptr(), w.data_ptr(), tiles.data_ptr(),
-                                   n_tiles.data_ptr(), max_tiles, out.data_ptr(), rows, E, hidden, inner))
+                                   n_tiles.data_ptr(), max_tiles, tile_rows, out.data_ptr(), rows, E, hidden, inner))
 
 
 def route_combine(y: torch.Tensor, row_of_pair, weights: torch.Tensor, residual: torch.Tensor) -> None:

@@ -50,20 +50,21 @@ def _declare(lib):
         "sp_sample_workspace_floats": [c_int, c_int],
         "sp_feed_tokens": [c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_random_fill": [c_void, c_int, c_void, c_i64, ctypes.c_uint64, c_i64, c_float, c_float, c_int],
-        "sp_layernorm": [c_void, c_void, c_void, c_int, c_void, c_float, c_int, c_void, c_int, c_int],
+        "sp_layernorm": [c_void, c_void, c_void, c_int, c_void, c_void, c_float, c_int, c_void, c_void, c_int, c_int],
         "sp_embed_bigram": [c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void,
                             c_int, c_int, c_int, c_int, c_int, c_int],
         "sp_latent_prepare": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_float,
                               c_void, c_void, c_int, c_float, c_int, c_void, c_void, c_void, c_int, c_int, c_void, c_int],
         "sp_head_gemm": [c_void, c_int, c_void, c_i64, c_i64, c_void, c_void, c_i64, c_i64, c_void, c_i64, c_int, c_int,
                          c_int, c_int],
-        "sp_group_tile_rows": [],
+        "sp_group_tile_rows": [c_int, c_i64, c_int, c_int],
         "sp_route_topk": [c_void, c_void, c_void, c_void, c_int, c_int, c_int],
         "sp_route_max_tiles": [c_int, c_int, c_int],
+        "sp_route": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_void, c_void, c_void],
         "sp_route_sort": [c_void, c_void, c_int, c_int, c_int, c_void, c_void, c_void, c_void],
-        "sp_expert_gate_up": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_void, c_int, c_int,
-                              c_int, c_int, c_int],
-        "sp_expert_down": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_int],
+        "sp_expert_gate_up": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_void, c_int, c_void, c_int,
+                              c_int, c_int, c_int, c_int],
+        "sp_expert_down": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_int],
         "sp_route_combine": [c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int],
         "sp_probe_read": [c_void, c_void, c_i64, c_int, c_void],
         "sp_probe_mfma": [c_void, c_int, c_int, c_void, ctypes.POINTER(ctypes.c_double)],

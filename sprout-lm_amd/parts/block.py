@@ -51,10 +51,14 @@ class ParallelBlock(Block):
     def forward(self, ctx, residual, caches):
         T, H = residual.shape
         h = ctx.buffer("normed", (T, H), ctx.act_dtype)
-        self.mixer_norm.forward(ctx, residual, h)
-        if self.ffn is not None:
+        if self.ffn is None:
+            self.mixer_norm.forward(ctx, residual, h)
+        else:
             h2 = ctx.buffer("normed_ffn", (T, H), ctx.act_dtype)
-            self.ffn_norm.forward(ctx, residual, h2)
+            pair = getattr(self.mixer_norm, "forward_pair", None)      # norms that share their statistics take one pass
+            if pair is None or not pair(ctx, self.ffn_norm, residual, h, h2):
+                self.mixer_norm.forward(ctx, residual, h)
+                self.ffn_norm.forward(ctx, residual, h2)
         self.mixer.forward(ctx, h, residual, caches.get("mixer"))
         if self.ffn is not None:
             self.ffn.forward(ctx, h2, residual)

@@ -83,7 +83,13 @@ class LatentAttention(Mixer):
         q, dkv, norm, uk, uv, g, o = self.names
         H = self.heads
         # one product for everything that reads the mixer's input: queries, latent + rotated key part, gates
-        self.w_in = torch.cat([tensors[q], tensors[dkv]] + ([tensors[g]] if self.gated else []), dim=0).contiguous()
+        # (rows of zeros behind them bring a row of results to a multiple of 8 numbers: every token's row, and with
+        # head sizes in eights every head's part of it, then starts at a multiple of 16 bytes for the per-head products)
+        stacked = [tensors[q], tensors[dkv]] + ([tensors[g]] if self.gated else [])
+        rows = sum(t.shape[0] for t in stacked)
+        if rows % 8:
+            stacked.append(torch.zeros(8 - rows % 8, self.hidden, dtype=tensors[q].dtype, device=tensors[q].device))
+        self.w_in = torch.cat(stacked, dim=0).contiguous()
         self.q_off, self.dkv_off = 0, H * (self.dim + self.rot_dim)
         self.gate_off = self.dkv_off + self.key_width
         self.w_norm = tensors[norm]

@@ -15,8 +15,8 @@ class RoutedExperts(FeedForward):
     """y = sum over a token's `top` experts of weight_e * down_e(act(gate_e x) * up_e x)  (+ shared(x)).
 
     Router logits z = W_r x + b are float32; the `top` largest are chosen (the lowest index wins a tie) and their
-    weights are the softmax over the chosen logits alone.  Nothing is decided on the host: a kernel sorts the
-    (token, choice) pairs by expert and cuts every expert's rows into tiles, the two grouped products walk those
+    weights are the softmax over the chosen logits alone.  Nothing is decided on the host: a kernel makes the choice,
+    sorts the (token, choice) pairs by expert and cuts every expert's rows into tiles, the two grouped products walk those
     tiles (the first gathers its rows from the tokens and applies the activation, the second writes float32 rows),
     and the weighted sum is taken per token in the order of its choices, so a token's result does not depend on what
     else is in the step.
@@ -86,16 +86,17 @@ class RoutedExperts(FeedForward):
         ops.gemm(h, self.w_router, logits, bias=self.b_router)
         ids = ctx.buffer("expert_ids", (T, top), torch.int32)
         weights = ctx.buffer("expert_weights", (T, top), torch.float32)
-        ops.route_topk(logits, ids, weights)
         row_of_pair = ctx.buffer("expert_row_of_pair", (pairs,), torch.int32)
         pair_of_row = ctx.buffer("expert_pair_of_row", (pairs,), torch.int32)
-        tiles = ctx.buffer("expert_tiles", (3 * ops.route_max_tiles(pairs, E),), torch.int32)
+        tile_rows = ops.group_tile_rows(ctx.act_dtype, pairs, E, self.hidden % 8 == 0 and self.inner % 8 == 0)
+        tiles = ctx.buffer("expert_tiles", (3 * ops.route_max_tiles(pairs, E, tile_rows),), torch.int32)
         n_tiles = ctx.buffer("expert_tile_count", (1,), torch.int32)
-        ops.route_sort(ids, E, row_of_pair, pair_of_row, tiles, n_tiles)
+        ops.route(logits, ids, weights, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
         act = ctx.buffer("expert_act", (pairs, self.inner), ctx.act_dtype)
-        ops.expert_gate_up(h, self.w_gate_up, tiles, n_tiles, pair_of_row, top, act, activation=self.activation)
+        ops.expert_gate_up(h, self.w_gate_up, tiles, n_tiles, pair_of_row, top, act, activation=self.activation,
+                           tile_rows=tile_rows)
         out = ctx.buffer("expert_out", (pairs, self.hidden), torch.float32)
-        ops.expert_down(act, self.w_down, tiles, n_tiles, out)
+        ops.expert_down(act, self.w_down, tiles, n_tiles, out, tile_rows=tile_rows)
         ops.route_combine(out, row_of_pair, weights, residual)
         if self.shared is not None:
             self.shared.forward(ctx, h, residual)

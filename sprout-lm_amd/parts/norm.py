@@ -47,3 +47,10 @@ class LayerNorm(Norm):
     def forward(self, ctx, x, out, rows=None):
         ops.layernorm(x, self.w[self.tensor], self.eps, out, rows)
         return out
+
+    def forward_pair(self, ctx, other, x, out, other_out) -> bool:
+        """This norm and `other` of the same x in one pass, where `other` differs in its weight alone."""
+        if not isinstance(other, LayerNorm) or other.size != self.size or other.eps != self.eps:
+            return False
+        ops.layernorm(x, self.w[self.tensor], self.eps, out, None, other.w[other.tensor], other_out)
+        return True

@@ -206,7 +206,11 @@ def moe(w, prefix: str, mlp: dict, h):
 
 def run_order(cfg):
     """(layer whose tensors run, the entry) for every layer of the list."""
-    return [(entry.get("weights_of", i), entry) for i, entry in enumerate(cfg["layers"])]
+    def owner(i):
+        while cfg["layers"][i].get("weights_of") is not None:      # a layer may name one that names a third
+            i = cfg["layers"][i]["weights_of"]
+        return i
+    return [(owner(i), entry) for i, entry in enumerate(cfg["layers"])]
 
 
 def forward(w, cfg, tokens, store=f32, rows=None, angle_dtype=np.float64, trace=None):
