@@ -18,6 +18,11 @@ part of a step that the host spends planning and launching, which the look-ahead
 `prefill_in_portions`: the same prompt prefilled 256 and 512 tokens a step; `mixed`: the batch decoding while
 another prompt is prefilled 256 tokens a step; with --pressure SHARE, the batch in a pool too small for its
 requests at the headline sizes.
+
+    python bench.py --design megozen [--sizes s,m,l] [--design-batches 1,8,64]
+
+times the Megozen presets instead (latent attention, routed experts), each beside the dense model of equal width,
+layers, vocabulary and work per token, and prints a line of its own; the default workload above is untouched.
 """
 from __future__ import annotations
 
@@ -275,8 +280,47 @@ def second_model_points(preset, dtype, element, batch, context, prefill_tokens, 
     return out
 
 
+def design_points(design: str, sizes: list[str], dtype: str, dtype_name: str, batches: list[int], context: int,
+                  prefill_tokens: int, steps: int, warmup: int, which: str = "both") -> dict:
+    """Decode and prefill throughput of another design's presets (`<design>-<size>`) beside the dense model of equal
+    width, layers, vocabulary and work per token (`<design>-<size>-dense`), random weights, every layer."""
+    import gc
+    import torch
+    from sprout_lm_amd.cli import PRESETS
+    from sprout_lm_amd.registry import config_from_dict
+    element = 2 if dtype_name == "bf16" else 4
+    out = {}
+    for size in sizes:
+        for name in ([f"{design}-{size}"] if which != "dense" else []) + ([f"{design}-{size}-dense"] if which != "design" else []):
+            gc.collect()
+            torch.cuda.empty_cache()
+            cfg = config_from_dict(dict(PRESETS[name]))
+            engine = make_engine(cfg, dtype, max(batches), context, prefill_tokens)
+            parts = engine.model.parts
+            point = {"weights_gb": round(parts.weight_bytes(element) / 1e9, 3),
+                     "cache_bytes_per_token": parts.cache_bytes_per_context_token(element)}
+            for batch in batches:
+                step_s, _ = measure_decode(engine, cfg, batch, context, steps, warmup)
+                point[f"decode_b{batch}_tok_s"] = round(batch / step_s, 1)
+                point[f"decode_b{batch}_ms"] = round(step_s * 1000, 4)
+            prefill_s = measure_prefill(engine, cfg, prefill_tokens, repeats=3)
+            point[f"prefill_{prefill_tokens}_tok_s"] = round(prefill_tokens / prefill_s, 1)
+            point[f"prefill_{prefill_tokens}_ms"] = round(prefill_s * 1000, 3)
+            point[f"prefill_{prefill_tokens}_frac_of_peak"] = round(prefill_flops(parts, prefill_tokens) / prefill_s / MFMA_PEAK[dtype_name], 5)
+            engine.close()
+            out[name] = point
+    return out
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
+    parser.add_argument("--design", default=None, choices=["megozen"],
+                        help="time nothing but this design's presets (--sizes) beside dense models of equal size: "
+                             "decode at --design-batches and --context, prefill of --prefill-tokens; prints a line of its own")
+    parser.add_argument("--sizes", default="s,m,l", help="with --design: which of its presets")
+    parser.add_argument("--design-batches", default="1,8,64", help="with --design: decode batch sizes")
+    parser.add_argument("--twin", default="both", choices=["both", "design", "dense"],
+                        help="with --design: time the design's presets, their dense twins, or both (for a profile of one)")
     parser.add_argument("--gpus", type=int, default=1)
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=8)
@@ -305,6 +349,16 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine does not run on {args.gpus} GPUs.")
         return 2
+
+    if args.design:
+        dtype = {"bf16": "bfloat16", "fp32": "float32"}[args.dtype]
+        points = design_points(args.design, [x for x in args.sizes.split(",") if x], dtype, args.dtype,
+                               [int(b) for b in args.design_batches.split(",")], args.context, args.prefill_tokens,
+                               args.steps, args.warmup, args.twin)
+        print(json.dumps({"metric": f"decode and prefill tok/s of {args.design} presets beside dense models of equal size",
+                          "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic", "context": args.context,
+                          "steps": args.steps, "warmup": args.warmup, "points": points}))
+        return 0
 
     from sprout_lm_amd.cli import PRESETS
     from sprout_lm_amd.registry import config_from_dict

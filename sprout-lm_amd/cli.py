@@ -43,6 +43,44 @@ PRESETS = {
 }
 
 
+def _megozen_preset(width: int, layers: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, experts: int,
+                    top: int, ff: int, shared_ff: int, window: int | None, vocab: int, own: int | None = None) -> dict:
+    """A Megozen configuration of `layers` equal layers, of which the first `own` have tensors (the others run with
+    those of layer i mod own)."""
+    mixer = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank,
+             "scale": (dim + rot_dim) ** -0.5,
+             "rot": {"base": 500000.0, "dims": rot_dim, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    if window:
+        mixer["mask"] = {"size": window}
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": ff}, "shared": {"ff": shared_ff}}
+    own = own or layers
+    entries = [dict({"type": "latent_attention", "mixer": mixer, "mlp": mlp}, **({"weights_of": i % own} if i >= own else {}))
+               for i in range(layers)]
+    return {"architecture": "Megozen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 8191, "mul_cur": 131}}, "layers": entries}
+
+
+def _dense_twin(width: int, layers: int, heads: int, kv_heads: int, inner: int, vocab: int) -> dict:
+    """The dense Qwen2 layer sizes that compute as much per token as a Megozen preset: the same width, layers and
+    vocabulary, `inner` = what a token's chosen experts and the shared one hold together."""
+    return dict(model_type="qwen2", hidden_act="silu", hidden_size=width, intermediate_size=inner, num_hidden_layers=layers,
+                num_attention_heads=heads, num_key_value_heads=kv_heads, vocab_size=vocab, max_position_embeddings=32768,
+                rms_norm_eps=1e-6, rope_theta=1000000.0, tie_word_embeddings=False, eos_token_id=0)
+
+
+PRESETS.update({
+    # small: 8 layers of width 1,024 (4 with tensors, each run twice), a window of 1,024 keys
+    "megozen-s": _megozen_preset(1024, 8, 8, 64, 32, 64, 96, 16, 2, 512, 1024, 1024, 32768, own=4),
+    "megozen-s-dense": _dense_twin(1024, 8, 8, 1, 2048, 32768),
+    # medium: 12 layers of width 2,048, every earlier key visible
+    "megozen-m": _megozen_preset(2048, 12, 16, 64, 32, 64, 96, 32, 4, 704, 1408, None, 32768),
+    "megozen-m-dense": _dense_twin(2048, 12, 16, 2, 4224, 32768),
+    # large: 8 layers of width 4,096, 32 heads over one latent
+    "megozen-l": _megozen_preset(4096, 8, 32, 64, 32, 64, 96, 64, 6, 1024, 2048, None, 32768),
+    "megozen-l-dense": _dense_twin(4096, 8, 32, 4, 8192, 32768),
+})
+
+
 def _env_int(name: str, default: int) -> int:
     value = os.environ.get(name)
     return default if value is None else int(value)

@@ -611,7 +611,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ decode_seqs,
     uint16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits, int nq,
-    int nkv, int page_size, int num_pages, int window, float scale2) {
+    int nkv, int kv_stored, int page_size, int num_pages, int window, float scale2) {
+  // nkv: the sets of query heads that a block takes at once (blockIdx.y); kv_stored: the key/value heads the pools
+  // hold.  They are the same unless a key/value head serves more query heads than the 16 rows of a block: then
+  // its heads are taken in nkv / kv_stored sets that read the same keys.
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   __shared__ float s_o[4][16][HD + 1];
   __shared__ float s_m[4][16], s_l[4][16];
@@ -647,9 +650,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   PagedKV kv;
   kv.page_size = page_size;
   kv.num_pages = num_pages;
-  kv.page_stride = size_t(nkv) * page_size * HD;
-  kv.k = k_pool + size_t(g) * page_size * HD;
-  kv.v = v_pool + size_t(g) * page_size * HD;
+  const int stored = g / (nkv / kv_stored);
+  kv.page_stride = size_t(kv_stored) * page_size * HD;
+  kv.k = k_pool + size_t(stored) * page_size * HD;
+  kv.v = v_pool + size_t(stored) * page_size * HD;
   kv.table = s_table;
   kv.table_first = table_first;
   kv.page_shift = page_shift;
@@ -896,7 +900,16 @@ bool attention_mfma_supports(int hd, int page_size, int nq, int nkv) {
   const bool hd_ok = hd % 16 == 0 && (dt <= 6 || dt == 8);
   return hd_ok && page_size % 4 == 0;
 }
-bool attention_mfma_decode_supports(int nq, int nkv) { return nq / nkv <= 16; }
+// A block of the one-query kernel holds up to 16 query heads; a key/value head that serves more is walked in sets
+// of the largest divisor of its heads that fits (20 heads: two sets of 10).
+static int decode_sets(int nq, int nkv) {
+  const int G = nq / nkv;
+  int rows = 1;
+  for (int d = 1; d <= 16; ++d)
+    if (G % d == 0) rows = d;
+  return nkv * (G / rows);
+}
+bool attention_mfma_decode_supports(int nq, int nkv) { return true; }
 int attention_mfma_tile_q(int hd) { return 32; }
 
 constexpr int kMaxPrefillSplits = 32;   // the merge kernel holds one split per lane; 64 would do as well
@@ -1024,13 +1037,13 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
     float* part_o = workspace;
     float* part_ml = workspace ? workspace + size_t(n_decode) * nq * n_splits * HD : nullptr;
     if ((page_size & (page_size - 1)) == 0)
-      attention_decode_kernel<DT, true><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+      attention_decode_kernel<DT, true><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
-          n_splits, nq, nkv, page_size, num_pages, window, scale2);
+          n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window, scale2);
     else
-      attention_decode_kernel<DT, false><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+      attention_decode_kernel<DT, false><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
-          n_splits, nq, nkv, page_size, num_pages, window, scale2);
+          n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window, scale2);
     if (check_launch("sp_attention (decode)")) return 1;
     if (n_splits > 1) {
       if (n_splits <= 16)
@@ -1098,13 +1111,15 @@ static int launch_decode_project(hipStream_t s, const void* q, int q_stride, con
   float* part_o = workspace;
   float* part_ml = workspace + size_t(n_decode) * nq * n_splits * HD;
   if ((page_size & (page_size - 1)) == 0)
-    attention_decode_kernel<DT, true><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+    attention_decode_kernel<DT, true><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
         (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
-        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, nkv, page_size, num_pages, window, scale * kLog2e);
+        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window,
+        scale * kLog2e);
   else
-    attention_decode_kernel<DT, false><<<dim3(n_splits, nkv, n_decode), 256, 0, s>>>(
+    attention_decode_kernel<DT, false><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
         (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
-        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, nkv, page_size, num_pages, window, scale * kLog2e);
+        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window,
+        scale * kLog2e);
   if (check_launch("sp_attention_decode_project (decode)")) return 1;
   const int tpw = project_tiles_per_wave(n_decode, nq, hidden);
   const dim3 grid(nq, (hidden + 64 * tpw - 1) / (64 * tpw), (n_decode + 15) / 16);

@@ -80,10 +80,22 @@ __host__ __device__ inline bool pipe_tile_of(const PipeTiles& tiles, int block, 
 // v_mfma_f32_32x32x2_f32 (k-slot l / 32 of MFMA e is element 4 (l / 32) + e of the eight that a 32-byte slice of a
 // row holds, for both operands): true float32 products and sums, no reduced-precision mode, 1/8 of the bfloat16
 // rate per byte, so this form is bound by the matrix cores and not by its fetches.
-template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB, typename TE = uint16_t>
+// The grouped form (GROUPED): every group (an expert) has weights of its own, w_group_stride elements apart, and
+// multiplies the rows that a list of tiles gives it: tiles [n][3] = (group, first row, rows) with at most BM rows
+// each and n in *n_tiles; row r of the list reads operand row gather[r] / gather_div and writes output row r.  Block
+// b takes tile b / tiles_n and weight tile b % tiles_n.
+struct PipeGroups {
+  const int32_t* tiles;
+  const int32_t* n_tiles;
+  const int32_t* gather;
+  int gather_div;
+  long long w_group_stride;
+};
+
+template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE, typename TB, typename TE = uint16_t, bool GROUPED = false>
 __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2 : 1)) void gemm_pipe_kernel(const TE* __restrict__ x, const TE* __restrict__ w,
                                                         const TB* __restrict__ bias, void* __restrict__ out, int T,
-                                                        int N, int K, int k_per_split, RopeArgs rope) {
+                                                        int N, int K, int k_per_split, RopeArgs rope, PipeGroups groups) {
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int ESZ = sizeof(TE), KSTEP = 128 / ESZ;    // elements of a tile row
   static_assert(ESZ == 2 || (MODE != kSilu && MODE != kRope && MODE != kStore), "float32 operands store or add float32");
@@ -103,24 +115,39 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N, (WAVES_M * WAVES_N <= 4 ? 2
   // whatever the number of tokens, and x stays in the caches.  The weight tiles left over when their number is no
   // multiple of 8 are dealt out by token tile, an equal run of their blocks to every XCD: four left-over weight
   // tiles would otherwise be a quarter more blocks on four of the XCDs, and fewer than 8 weight tiles idle XCDs.
-  const PipeTiles tiles = pipe_tiles((T + BM - 1) / BM, ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
-  int tile_n, tile_t;
-  if (!pipe_tile_of(tiles, blockIdx.x, &tile_t, &tile_n)) return;
-  const int t0 = tile_t * BM, n0 = tile_n * BN;
+  int tile_n, tile_t, t0;
+  if constexpr (GROUPED) {
+    const int tiles_n = ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN;
+    tile_t = blockIdx.x / tiles_n;
+    tile_n = blockIdx.x - tile_t * tiles_n;
+    if (tile_t >= *groups.n_tiles) return;
+    w += groups.tiles[3 * tile_t] * groups.w_group_stride;
+    t0 = groups.tiles[3 * tile_t + 1];
+    T = t0 + groups.tiles[3 * tile_t + 2];      // the tile's rows end here
+  } else {
+    const PipeTiles tiles = pipe_tiles((T + BM - 1) / BM, ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
+    if (!pipe_tile_of(tiles, blockIdx.x, &tile_t, &tile_n)) return;
+    t0 = tile_t * BM;
+  }
+  const int n0 = tile_n * BN;
   const int k_begin = blockIdx.z * k_per_split, k_end = min(K, k_begin + k_per_split);
   const int steps = (k_end - k_begin) / KSTEP;
   typedef __attribute__((address_space(3))) unsigned char* lds_address_t;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_address_t)pipe_lds;   // the tiles' offset within the LDS
 
   // ---- what this lane fetches: row 8 (NW j + wave) + lane / 8 of each operand tile, for j < LX (LW)
-  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(x + size_t(t0) * K + k_begin);
+  const unsigned char* xbase = reinterpret_cast<const unsigned char*>(x + (GROUPED ? size_t(0) : size_t(t0) * K) + k_begin);
   const unsigned char* wbase = reinterpret_cast<const unsigned char*>(w + (MODE == kSilu || MODE == kRope ? size_t(0) : size_t(n0) * K) + k_begin);
   uint32_t xoff[LX], woff[LW];
 #pragma unroll
   for (int j = 0; j < LX; ++j) {
     const int r = 8 * (NW * j + wave) + (lane >> 3);
     const int piece = (lane & 7) ^ swz(r);
-    xoff[j] = uint32_t(min(r, T - 1 - t0)) * uint32_t(K) * uint32_t(ESZ) + piece * 16;
+    if constexpr (GROUPED)
+      xoff[j] = uint32_t(groups.gather ? groups.gather[t0 + min(r, T - 1 - t0)] / groups.gather_div : t0 + min(r, T - 1 - t0)) *
+                    uint32_t(K) * uint32_t(ESZ) + piece * 16;
+    else
+      xoff[j] = uint32_t(min(r, T - 1 - t0)) * uint32_t(K) * uint32_t(ESZ) + piece * 16;
   }
 #pragma unroll
   for (int j = 0; j < LW; ++j) {
@@ -239,8 +266,31 @@ inline int launch_pipe_mode(hipStream_t s, int splits, const TE* x, const TE* w,
   // the kernel's own numbering of tiles
   const PipeTiles tiles = pipe_tiles((T + BM - 1) / BM, ((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
   dim3 grid(8 * (tiles.own + tiles.run), 1, splits);
-  gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB, TE><<<grid, 64 * WAVES_M * WAVES_N, lds, s>>>(x, w, bias, out, T, N, K, k_per_split, rope);
+  gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, TB, TE><<<grid, 64 * WAVES_M * WAVES_N, lds, s>>>(x, w, bias, out, T, N, K, k_per_split, rope, PipeGroups{});
   return check_launch("sp_gemm (pipelined)");
+}
+
+// The grouped form over `max_tiles` tiles of at most BM rows (see PipeGroups); K a multiple of 64, no split of K.
+template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE>
+inline int launch_pipe_grouped(hipStream_t s, const uint16_t* x, const uint16_t* w, void* out, int N, int K, int max_tiles,
+                               const PipeGroups& groups, const char* what) {
+  constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
+  constexpr size_t lds = size_t(STAGES) * (BM + BN) * 128;
+  static bool raised = false;
+  if (lds > 48 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, bf16_t, uint16_t, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
+    if (e != hipSuccess) {
+      set_error("%s: cannot raise the LDS limit: %s", what, hipGetErrorString(e));
+      return 1;
+    }
+    raised = true;
+  }
+  const long long blocks = (long long)max_tiles * (((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
+  SP_REQUIRE(blocks < (1ll << 31), "%s: too many tiles", what);
+  gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, bf16_t, uint16_t, true><<<dim3((unsigned)blocks), 64 * WAVES_M * WAVES_N, lds, s>>>(
+      x, w, nullptr, out, 0, N, K, K, RopeArgs{}, groups);
+  return check_launch(what);
 }
 
 

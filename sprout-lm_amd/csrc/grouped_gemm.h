@@ -29,8 +29,14 @@ enum { kStore = 0, kGated = 1, kSigmoid = 2 };
 // Whether the matrix-core kernels take these operands: bfloat16, K in whole groups of 8, and every row of a and w
 // starting at a multiple of 16 bytes.
 bool grouped_mfma_takes(int dtype, const GroupedArgs& p);
-// tile_rows: 64 or 128 rows a tile (with a tile list: the size the list was cut for).
+// tile_rows: 16, 64, 128 or 256 rows a tile (with a tile list: the size the list was cut for).
 int launch_grouped_mfma(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, int tile_rows,
                         const char* what);
+
+// The pipelined tiled kernel in its grouped form (grouped_gemm_pipe.hip): tiles of 128 or 256 rows from a tile list,
+// K in whole steps of 64, bfloat16; `gated`: SiLU(gate) * up into bfloat16, else a float32 store.
+int grouped_pipe(hipStream_t s, bool gated, const void* x, const void* w, long long w_group_stride, const int32_t* tiles,
+                 const int32_t* n_tiles, int max_tiles, int tile_rows, const int32_t* gather, int gather_div, void* out,
+                 int N, int K, const char* what);
 
 }  // namespace sprout

@@ -109,16 +109,28 @@ static int launch_grouped(hipStream_t s, int dtype, int out_dtype, const Grouped
 
 using namespace sprout;
 
-// Rows a tile of the grouped products holds: 128 where a group brings at least that many rows and the matrix-core
-// kernels take the sizes (bfloat16, K in eights), else 64.
+// Rows a tile of the grouped products holds.  Where the matrix-core kernels take the operands (bfloat16, K in
+// eights): 16 where a group has at most 8 rows on average (decoded tokens), 256 from 192 on, 128 from 96 on; 64 in
+// between and for every other operand.
 extern "C" int sp_group_tile_rows(int dtype, long long rows, int groups, int K) {
-  return (dtype == kBF16 && K % 8 == 0 && groups > 0 && rows / groups >= 128) ? 128 : GT;
+  if (dtype != kBF16 || K % 8 || groups <= 0) return GT;
+  const long long each = rows / groups;
+  if (rows <= 8ll * groups) return 16;
+  return each >= 192 ? 256 : each >= 96 ? 128 : GT;
 }
 
 // The float32-arithmetic kernel cuts its own tiles of 64 rows; a list cut for more rows is not for it.
 static int grouped(hipStream_t s, int mode, int dtype, int out_dtype, const GroupedArgs& p, int tiles, int tile_rows,
                    const char* what) {
-  if (grouped_mfma_takes(dtype, p)) return launch_grouped_mfma(s, mode, out_dtype, p, tiles, tile_rows, what);
+  if (grouped_mfma_takes(dtype, p)) {
+    // many rows a group, from a tile list: the pipelined tiled kernel (its two epilogues are the experts')
+    if (p.tiles && tile_rows >= 128 && p.K % 64 == 0 && p.a_group_stride == 0 && p.a_stride == p.K &&
+        ((mode == kGated && out_dtype == kBF16 && p.up_offset == p.N && p.out_stride == p.N) ||
+         (mode == kStore && out_dtype == kF32 && p.out_stride == p.N)) && p.out_group_stride == 0)
+      return grouped_pipe(s, mode == kGated, p.a, p.w, p.w_group_stride, p.tiles, p.n_tiles, tiles, tile_rows, p.gather,
+                          p.gather_div, p.out, p.N, p.K, what);
+    return launch_grouped_mfma(s, mode, out_dtype, p, tiles, tile_rows, what);
+  }
   SP_REQUIRE(tile_rows == GT, "%s: tiles of %d rows need operands the matrix-core kernels take", what, tile_rows);
   if (mode == kGated) return launch_grouped<kGated>(s, dtype, out_dtype, p, tiles, what);
   if (mode == kSigmoid) return launch_grouped<kSigmoid>(s, dtype, out_dtype, p, tiles, what);
@@ -140,7 +152,7 @@ extern "C" int sp_head_gemm(void* stream, int dtype, const void* a, long long a_
   p.gate = gate; p.gate_stride = gate_stride;
   p.rows = T;
   p.N = N; p.K = K;
-  const int tile_rows = (grouped_mfma_takes(dtype, p) && T >= 256) ? 128 : GT;
+  const int tile_rows = !grouped_mfma_takes(dtype, p) ? GT : T <= 32 ? 16 : T >= 256 ? 128 : GT;
   p.tiles_per_group = (T + tile_rows - 1) / tile_rows;
   const long long blocks = (long long)heads * p.tiles_per_group;
   SP_REQUIRE(blocks < (1ll << 31), "sp_head_gemm: too many tiles");

@@ -137,6 +137,86 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(GroupedArgs p) {
     }
 }
 
+// Few rows a tile (decoded tokens): tiles of up to 16 rows, a block per tile and 16 columns.  Nothing goes through
+// LDS on the way in: a lane takes its 16 bytes of a weight row and of an operand row straight from memory, four
+// steps of 32 along K at once (256 bytes of a row), and the four waves of a block take turns along K, so that a
+// product of one row against a whole expert is spread over hundreds of blocks with 64 KB on their way each.  The
+// operand rows are the A side of 16x16x32 MFMA tiles; the waves' sums are joined in LDS in a fixed order.
+template <int MODE, typename TO>
+__global__ __launch_bounds__(256) void grouped_skinny_kernel(GroupedArgs p) {
+  constexpr bool GATED = MODE == kGated;
+  constexpr int U = 4;
+  __shared__ float s_acc[3][64][GATED ? 8 : 4];
+  int group, row0, nrows;
+  if (p.tiles) {
+    if (int(blockIdx.x) >= *p.n_tiles) return;
+    group = p.tiles[3 * blockIdx.x];
+    row0 = p.tiles[3 * blockIdx.x + 1];
+    nrows = p.tiles[3 * blockIdx.x + 2];
+  } else {
+    group = blockIdx.x / p.tiles_per_group;
+    row0 = (blockIdx.x - group * p.tiles_per_group) * 16;
+    nrows = min(16, p.rows - row0);
+  }
+  const int n0 = blockIdx.y * 16;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 15, lj = lane >> 4;
+  const uint16_t* a_ptr = nullptr;
+  if (lr < nrows) {
+    const long long src = p.gather ? p.gather[row0 + lr] / p.gather_div : row0 + lr;
+    a_ptr = (const uint16_t*)p.a + src * p.a_stride + group * p.a_group_stride + 8 * lj;
+  }
+  const int n = n0 + lr;
+  const uint16_t* base = (const uint16_t*)p.w + group * p.w_group_stride + 8 * lj;
+  const uint16_t* w_ptr = n < p.N ? base + (long long)n * p.K : nullptr;
+  const uint16_t* u_ptr = (GATED && n < p.N) ? base + (long long)(p.up_offset + n) * p.K : nullptr;
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = wave * 32 * U; k0 < p.K; k0 += 4 * 32 * U) {
+    uint4 av[U], wv[U], uv[GATED ? U : 1];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + 32 * u;
+      const bool in_k = k + 8 * lj < p.K;
+      wv[u] = (w_ptr && in_k) ? ldg128(w_ptr + k) : zero;
+      if (GATED) uv[u] = (u_ptr && in_k) ? ldg128(u_ptr + k) : zero;
+      av[u] = (a_ptr && in_k) ? ldg128(a_ptr + k) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      acc = mfma16(as_bf16x8(av[u]), as_bf16x8(wv[u]), acc);
+      if (GATED) acc2 = mfma16(as_bf16x8(av[u]), as_bf16x8(uv[u]), acc2);
+    }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      s_acc[wave - 1][lane][r] = acc[r];
+      if (GATED) s_acc[wave - 1][lane][4 + r] = acc2[r];
+    }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int w = 0; w < 3; ++w)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      acc[r] += s_acc[w][lane][r];
+      if (GATED) acc2[r] += s_acc[w][lane][4 + r];
+    }
+  // lane l, number r: row 4 (l / 16) + r, column l % 16
+  if (n >= p.N) return;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = 4 * lj + r;
+    if (row >= nrows) continue;
+    float v = acc[r];
+    if (GATED) v = (v / (1.0f + expf(-v))) * acc2[r];
+    if (MODE == kSigmoid)
+      v *= 1.0f / (1.0f + expf(-to_float(((const bf16_t*)p.gate)[(long long)(row0 + row) * p.gate_stride + group])));
+    ((TO*)p.out)[(long long)(row0 + row) * p.out_stride + group * p.out_group_stride + n] = from_float<TO>(v);
+  }
+}
+
 bool grouped_mfma_takes(int dtype, const GroupedArgs& p) {
   auto whole = [](long long n) { return n % 8 == 0; };
   return dtype == kBF16 && p.K > 0 && whole(p.K) && whole(p.a_stride) && whole(p.a_group_stride) && whole(p.w_group_stride) &&
@@ -154,11 +234,26 @@ static int launch_shape(hipStream_t s, int mode, int out_dtype, const GroupedArg
   return check_launch(what);
 }
 
+static int launch_skinny(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, const char* what) {
+  dim3 grid(tiles, (p.N + 15) / 16);
+  if (mode == kStore && out_dtype == kBF16) grouped_skinny_kernel<kStore, bf16_t><<<grid, 256, 0, s>>>(p);
+  else if (mode == kStore && out_dtype == kF32) grouped_skinny_kernel<kStore, float><<<grid, 256, 0, s>>>(p);
+  else if (mode == kGated && out_dtype == kBF16) grouped_skinny_kernel<kGated, bf16_t><<<grid, 256, 0, s>>>(p);
+  else if (mode == kSigmoid && out_dtype == kBF16) grouped_skinny_kernel<kSigmoid, bf16_t><<<grid, 256, 0, s>>>(p);
+  else SP_REQUIRE(false, "%s: no matrix-core kernel for epilogue %d with output type %d", what, mode, out_dtype);
+  return check_launch(what);
+}
+
 int launch_grouped_mfma(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, int tile_rows,
                         const char* what) {
-  SP_REQUIRE(tile_rows == 64 || tile_rows == 128, "%s: tiles of %d rows", what, tile_rows);
-  // wide tiles where there are columns for them; the gated epilogue keeps two sets of accumulators
+  SP_REQUIRE(tile_rows == 16 || tile_rows == 64 || tile_rows == 128 || tile_rows == 256, "%s: tiles of %d rows", what, tile_rows);
+  if (tile_rows == 16) return launch_skinny(s, mode, out_dtype, p, tiles, what);
+  // wide tiles where there are columns for them; the gated epilogue keeps two sets of accumulators, so its tiles of
+  // 256 rows are narrow.  Tiles of 256 rows hold a group's rows in one block where they can: its weights are then
+  // fetched once, not once per tile.
   const bool wide = p.N > 64;
+  if (tile_rows == 256) return (wide && mode != kGated) ? launch_shape<256, 128>(s, mode, out_dtype, p, tiles, what)
+                                                        : launch_shape<256, 64>(s, mode, out_dtype, p, tiles, what);
   if (tile_rows == 128) return wide ? launch_shape<128, 128>(s, mode, out_dtype, p, tiles, what)
                                     : launch_shape<128, 64>(s, mode, out_dtype, p, tiles, what);
   return wide ? launch_shape<64, 128>(s, mode, out_dtype, p, tiles, what)

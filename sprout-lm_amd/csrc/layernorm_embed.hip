@@ -15,6 +15,36 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int32_t* __r
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const float* in = x + size_t(rows ? rows[r] : r) * H;
+  TO* o = out + size_t(r) * H;
+  TO* o2 = out2 ? out2 + size_t(r) * H : nullptr;
+  constexpr int KEEP = 8;
+  if (H <= KEEP * int(blockDim.x)) {      // the row stays in registers: one trip to memory
+    float v[KEEP];
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < KEEP; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      v[j] = i < H ? in[i] : 0.f;
+      sum += v[j];
+    }
+    const float mean = block_sum(sum, scratch) / float(H);
+    float sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < KEEP; ++j) {
+      const float d = threadIdx.x + j * blockDim.x < H ? v[j] - mean : 0.f;
+      sq = fmaf(d, d, sq);
+    }
+    const float scale = 1.0f / sqrtf(block_sum(sq, scratch) / float(H) + eps);
+#pragma unroll
+    for (int j = 0; j < KEEP; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      if (i >= H) continue;
+      const float y = (v[j] - mean) * scale;
+      o[i] = from_float<TO>(y * to_float(w[i]));
+      if (o2) o2[i] = from_float<TO>(y * to_float(w2[i]));
+    }
+    return;
+  }
   float sum = 0.f;
   for (int i = threadIdx.x; i < H; i += blockDim.x) sum += in[i];
   const float mean = block_sum(sum, scratch) / float(H);
@@ -24,8 +54,6 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int32_t* __r
     sq = fmaf(d, d, sq);
   }
   const float scale = 1.0f / sqrtf(block_sum(sq, scratch) / float(H) + eps);
-  TO* o = out + size_t(r) * H;
-  TO* o2 = out2 ? out2 + size_t(r) * H : nullptr;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     const float y = (in[i] - mean) * scale;
     o[i] = from_float<TO>(y * to_float(w[i]));

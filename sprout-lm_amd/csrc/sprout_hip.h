@@ -209,7 +209,7 @@ int sp_expert_gate_up(void* stream, int dtype, const void* x, const void* w, con
                       int inner, int K, int activation);
 int sp_expert_down(void* stream, int dtype, const void* act, const void* w, const int32_t* tiles, const int32_t* n_tiles,
                    int max_tiles, int tile_rows, float* out, int rows, int experts, int hidden, int inner);
-// sp_route: sp_route_topk and sp_route_sort in one call (one launch up to 8,192 tokens).
+// sp_route: sp_route_topk and sp_route_sort in one call (one launch up to 256 tokens).
 int sp_route(void* stream, const float* logits, int32_t* ids, float* weights, int T, int experts, int top, int tile_rows,
              int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
 int sp_route_combine(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,

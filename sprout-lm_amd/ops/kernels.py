@@ -240,7 +240,7 @@ def route_topk(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -
 
 def route(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, row_of_pair, pair_of_row, tiles, n_tiles,
           tile_rows: int = 64) -> None:
-    """route_topk and route_sort in one call (one launch for steps of up to 8,192 tokens)."""
+    """route_topk and route_sort in one call (one launch for steps of up to 256 tokens)."""
     _gpu(logits, "router logits"); _gpu(ids, "chosen experts"); _gpu(weights, "expert weights")
     T, E = logits.shape
     top = ids.shape[1]

@@ -264,7 +264,7 @@ def test_router_choice_ties_and_weights():
         n_tiles = torch.zeros(1, dtype=torch.int32, device=DEV)
         ops.route_sort(ids, E, row_of_pair, pair_of_row, tiles, n_tiles)
         # choice and order in one call, for tiles of either size
-        for tile_rows in (64, 128):
+        for tile_rows in (16, 64, 128, 256):
             ids2, weights2 = torch.empty_like(ids), torch.empty_like(weights)
             rp2, pr2 = torch.empty_like(row_of_pair), torch.empty_like(pair_of_row)
             tiles2 = torch.full((3 * ops.route_max_tiles(pairs, E, tile_rows),), -7, dtype=torch.int32, device=DEV)
