@@ -87,7 +87,8 @@ __global__ void embed_bigram_kernel(const TW* __restrict__ table, const TW* __re
     } else {
       previous = tokens[t - 1];
     }
-    if (positions[t] > 0) row = ((long long)previous * mul_prev + (long long)cur * mul_cur) % buckets;
+    // (a * m) mod b = (a * (m mod b)) mod b: with the multipliers reduced first the products stay far inside 64 bits
+    if (positions[t] > 0) row = (((long long)previous * (mul_prev % buckets)) % buckets + ((long long)cur * (mul_cur % buckets)) % buckets) % buckets;
     row_s = row;
   }
   __syncthreads();
@@ -122,10 +123,10 @@ extern "C" int sp_layernorm(void* stream, const float* x, const int32_t* rows, i
 extern "C" int sp_embed_bigram(void* stream, int table_dtype, const void* table, const void* pairs,
                                const int32_t* tokens, const int32_t* positions, const int32_t* q_start,
                                const int32_t* q_len, const int32_t* seq_of_token, const int32_t* state_slots,
-                               int32_t* last_token, float* residual, int T, int H, int V, int buckets, int mul_prev,
-                               int mul_cur) {
+                               int32_t* last_token, float* residual, int T, int H, int V, long long buckets,
+                               long long mul_prev, long long mul_cur) {
   SP_REQUIRE(T >= 0 && H > 0 && V > 0 && buckets > 0 && mul_prev >= 0 && mul_cur >= 0,
-             "sp_embed_bigram: bad sizes T=%d H=%d V=%d buckets=%d", T, H, V, buckets);
+             "sp_embed_bigram: bad sizes T=%d H=%d V=%d buckets=%lld", T, H, V, buckets);
   SP_REQUIRE(table && pairs && tokens && positions && q_start && q_len && seq_of_token && state_slots && last_token &&
                  residual, "sp_embed_bigram: null operand");
   if (T == 0) return 0;

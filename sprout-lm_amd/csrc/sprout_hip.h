@@ -166,8 +166,8 @@ int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype,
 // is left for the next step.
 int sp_embed_bigram(void* stream, int table_dtype, const void* table, const void* pairs, const int32_t* tokens,
                     const int32_t* positions, const int32_t* q_start, const int32_t* q_len, const int32_t* seq_of_token,
-                    const int32_t* state_slots, int32_t* last_token, float* residual, int T, int H, int V, int buckets,
-                    int mul_prev, int mul_cur);
+                    const int32_t* state_slots, int32_t* last_token, float* residual, int T, int H, int V,
+                    long long buckets, long long mul_prev, long long mul_cur);
 
 // Attention over a latent, between the input projections and the attention kernel.  A row of proj holds per head
 // [dim unrotated, rot rotated] query numbers from column q_off on, and at dkv_off the latent (rank numbers) and

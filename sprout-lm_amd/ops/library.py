@@ -52,7 +52,7 @@ def _declare(lib):
         "sp_random_fill": [c_void, c_int, c_void, c_i64, ctypes.c_uint64, c_i64, c_float, c_float, c_int],
         "sp_layernorm": [c_void, c_void, c_void, c_int, c_void, c_void, c_float, c_int, c_void, c_void, c_int, c_int],
         "sp_embed_bigram": [c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void,
-                            c_int, c_int, c_int, c_int, c_int, c_int],
+                            c_int, c_int, c_int, c_i64, c_i64, c_i64],
         "sp_latent_prepare": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_float,
                               c_void, c_void, c_int, c_float, c_int, c_void, c_void, c_void, c_int, c_int, c_void, c_int],
         "sp_head_gemm": [c_void, c_int, c_void, c_i64, c_i64, c_void, c_void, c_i64, c_i64, c_void, c_i64, c_int, c_int,

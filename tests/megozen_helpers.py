@@ -62,9 +62,18 @@ ONE_LAYER = model(64, 150, [layer(mixer(2, 16, 8, 16, 24, 0.5, window=29), exper
 ALL_CHOSEN = model(96, 211, [layer(_G, experts(3, 3, 32, shared=24)), layer(_G, experts(3, 3, 32, shared=24)),
                              layer(_G, experts(3, 3, 32, shared=24), weights_of=0)])
 
-CONFIGS = {"general": GENERAL, "varied": VARIED, "many_heads": MANY_HEADS, "one_layer": ONE_LAYER, "all_chosen": ALL_CHOSEN}
-PAGE = {"general": 16, "varied": 16, "many_heads": 8, "one_layer": 4, "all_chosen": 16}
-SEED = {"general": 5, "varied": 6, "many_heads": 7, "one_layer": 8, "all_chosen": 9}
+# sizes in no whole eights or sixteens anywhere (width 100, key width 22, head sizes 12 + 6, values of 10, experts of 28
+# and 36); a window of one key, a window of five inside a page, and a layer that sees everything; a router without a
+# shared expert beside one with; large multipliers in the pair table
+_O1 = mixer(5, 12, 6, 10, 16, 0.7, window=1, base=300.0)
+_O5 = mixer(5, 12, 6, 10, 16, 0.7, window=5, scaling=(3.0, 16, 4.0, 1.0))
+_OA = mixer(3, 20, 2, 6, 30, 0.2, window=None, base=20.0, scaling=(1.5, 8, 2.0, 1.0))
+ODD = model(100, 77, [layer(_O1, experts(3, 2, 28)), layer(_O5, experts(9, 4, 36, shared=28)), layer(_OA),
+                      layer(_O5, experts(9, 4, 36, shared=28), weights_of=1)], bigram=(13, 2 ** 31 + 11, 2 ** 20 + 3), eps=1e-3)
+
+CONFIGS = {"odd": ODD, "general": GENERAL, "varied": VARIED, "many_heads": MANY_HEADS, "one_layer": ONE_LAYER, "all_chosen": ALL_CHOSEN}
+PAGE = {"odd": 16, "general": 16, "varied": 16, "many_heads": 8, "one_layer": 4, "all_chosen": 16}
+SEED = {"odd": 4, "general": 5, "varied": 6, "many_heads": 7, "one_layer": 8, "all_chosen": 9}
 
 
 def random_weights(cfg: dict, seed: int) -> dict:

@@ -109,7 +109,8 @@ def test_layer_norm(dtype, H):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("vocab,buckets,mul_prev,mul_cur", [(150, 97, 31, 5), (40, 1, 0, 0), (300, 64, 3, 1),
-                                                          (60000, 1013, 40009, 77003), (90, 7, 0, 3), (90, 11, 5, 0)])
+                                                          (60000, 1013, 40009, 77003), (90, 7, 0, 3), (90, 11, 5, 0),
+                                                          (500, 1013, 2 ** 40 + 7, 2 ** 35 + 1)])
 def test_bigram_embedding_across_steps_and_reused_slots(dtype, vocab, buckets, mul_prev, mul_cur):
     """Sequences fed in portions and single tokens beside each other; the token before a portion comes from the
     request's state slot; a slot given back serves the next request, whose first token takes the last row.  The
@@ -483,7 +484,7 @@ def check(folder, dtype, requests, trace, results):
     return worst
 
 
-LENGTHS = {"general": [1, 9, 40, 97, 130, 33, 2, 75], "varied": [48, 150, 65, 90, 33, 3], "many_heads": [5, 17, 70, 64, 40],
+LENGTHS = {"odd": [1, 2, 21, 70, 45, 97], "general": [1, 9, 40, 97, 130, 33, 2, 75], "varied": [48, 150, 65, 90, 33, 3], "many_heads": [5, 17, 70, 64, 40],
            "one_layer": [2, 70, 97, 33, 64, 120], "all_chosen": [9, 40, 97, 33, 110]}
 # bfloat16 where rounding cannot flip an expert between the two sides: one layer (both sides route the same stored
 # input), or every expert chosen
