@@ -2,7 +2,7 @@
 
     python -m sprout_lm_amd demo [--json] [--pressure]
     python -m sprout_lm_amd generate MODEL_DIR --prompt-ids 1,2,3 [--max-new-tokens N] ...
-    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b | --config FILE  --out DIR [--seed N]
+    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b|megozen-s|... | --config FILE  --out DIR [--seed N]
 
 `demo` is the counterpart of the reference's src/demo.ts, with the reference's two options: a few requests on a
 tiny random model, told round by round (--json: the same as one JSON document; --pressure: a pool so small that
