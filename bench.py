@@ -6,7 +6,7 @@
 Default: Qwen2.5-0.5B layer sizes with random weights, bfloat16, a batch
 of 8 requests at a context of 4,096 tokens.  A step is one decode step of the whole engine loop
 (scheduler, one batched model step, sampling, token ids back on the host).  Prints ONE JSON line.
-Beside the contract's fields the line holds the prefill of 2,048 tokens (the median of its repeats), the
+Beside the fields every such line must hold, it holds the prefill of 2,048 tokens (the median of its repeats), the
 roofline of the decode step, and `points`: decoding at batch 1, 64, 128 and 256, and the same decode step and
 prefill at Qwen2.5-7B and Qwen2.5-32B sizes with all their layers, each with its fraction of the published peak
 (`7b_...`, `32b_...`); at 32B sizes also the batch in a pool of 0.6 of the pages it needs (`32b_pressure_...`:

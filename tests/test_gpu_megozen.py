@@ -306,7 +306,7 @@ def expert_weights(rng, hidden, inner, experts, shared, dtype, bias=True):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("hidden,inner,experts,top,shared", [(40, 48, 5, 2, 24), (64, 24, 4, 4, None), (72, 40, 6, 1, 72),
-                                                            (128, 64, 16, 3, 32), (256, 128, 9, 2, 192)])
+                                                            (128, 64, 16, 3, 32), (256, 128, 9, 2, 192), (100, 36, 9, 4, 28)])
 @pytest.mark.parametrize("T", [1, 7, 150, 1100])
 def test_routed_experts_part(dtype, hidden, inner, experts, top, shared, T):
     """The feed-forward alone: one token (most experts get no row), a handful, more than a tile per expert, and enough
