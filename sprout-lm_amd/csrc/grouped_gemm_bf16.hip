@@ -138,14 +138,13 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(GroupedArgs p) {
 }
 
 // Few rows a tile (decoded tokens): tiles of up to 16 rows, a block per tile and 16 columns.  Nothing goes through
-// LDS on the way in: a lane takes its 16 bytes of a weight row and of an operand row straight from memory, four
-// steps of 32 along K at once (256 bytes of a row), and the four waves of a block take turns along K, so that a
+// LDS on the way in: a lane takes its 16 bytes of a weight row and of an operand row straight from memory, U = four
+// or (long K) eight steps of 32 along K at once (256 or 512 bytes of a row), and the four waves of a block take turns along K, so that a
 // product of one row against a whole expert is spread over hundreds of blocks with 64 KB on their way each.  The
 // operand rows are the A side of 16x16x32 MFMA tiles; the waves' sums are joined in LDS in a fixed order.
-template <int MODE, typename TO>
+template <int MODE, typename TO, int U>
 __global__ __launch_bounds__(256) void grouped_skinny_kernel(GroupedArgs p) {
   constexpr bool GATED = MODE == kGated;
-  constexpr int U = 4;
   __shared__ float s_acc[3][64][GATED ? 8 : 4];
   int group, row0, nrows;
   if (p.tiles) {
@@ -234,14 +233,20 @@ static int launch_shape(hipStream_t s, int mode, int out_dtype, const GroupedArg
   return check_launch(what);
 }
 
-static int launch_skinny(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, const char* what) {
+template <int U>
+static int launch_skinny_u(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, const char* what) {
   dim3 grid(tiles, (p.N + 15) / 16);
-  if (mode == kStore && out_dtype == kBF16) grouped_skinny_kernel<kStore, bf16_t><<<grid, 256, 0, s>>>(p);
-  else if (mode == kStore && out_dtype == kF32) grouped_skinny_kernel<kStore, float><<<grid, 256, 0, s>>>(p);
-  else if (mode == kGated && out_dtype == kBF16) grouped_skinny_kernel<kGated, bf16_t><<<grid, 256, 0, s>>>(p);
-  else if (mode == kSigmoid && out_dtype == kBF16) grouped_skinny_kernel<kSigmoid, bf16_t><<<grid, 256, 0, s>>>(p);
+  if (mode == kStore && out_dtype == kBF16) grouped_skinny_kernel<kStore, bf16_t, U><<<grid, 256, 0, s>>>(p);
+  else if (mode == kStore && out_dtype == kF32) grouped_skinny_kernel<kStore, float, U><<<grid, 256, 0, s>>>(p);
+  else if (mode == kGated && out_dtype == kBF16) grouped_skinny_kernel<kGated, bf16_t, U><<<grid, 256, 0, s>>>(p);
+  else if (mode == kSigmoid && out_dtype == kBF16) grouped_skinny_kernel<kSigmoid, bf16_t, U><<<grid, 256, 0, s>>>(p);
   else SP_REQUIRE(false, "%s: no matrix-core kernel for epilogue %d with output type %d", what, mode, out_dtype);
   return check_launch(what);
+}
+
+static int launch_skinny(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, const char* what) {
+  // a wave's turn along K is 32 U numbers: eight steps at once where K gives every wave two turns of them
+  return p.K >= 2048 ? launch_skinny_u<8>(s, mode, out_dtype, p, tiles, what) : launch_skinny_u<4>(s, mode, out_dtype, p, tiles, what);
 }
 
 int launch_grouped_mfma(hipStream_t s, int mode, int out_dtype, const GroupedArgs& p, int tiles, int tile_rows,
