@@ -388,11 +388,14 @@ def test_latent_attention_part(dtype, shape, schedule, spiky):
     assert sorted(part.tensors()) == sorted(w)
     part.bind({k: dev(v, dtype) for k, v in w.items()})
     part.prepare(DEV, dtype)
-    lengths = [150, 61]
+    # without a window the first sequence is long enough for several chunks of the one-query kernel, with flagged
+    # keys hundreds of places back and on both sides of a chunk's border
+    lengths = [150 if window else 600, 61]
     hs = [rng.standard_normal((n, hidden)) for n in lengths]
     if spiky:
         reach = window or 100
-        for h, flagged in zip(hs, ([0, 2 * page - 1, 2 * page, 149 - reach, 150 - reach, 90], [7, 60 - reach if reach < 60 else 8])):
+        far = [] if window else [3, 255, 256, 511, 512]
+        for h, flagged in zip(hs, ([0, 2 * page - 1, 2 * page, 149 - reach, 150 - reach, 90] + far, [7, 60 - reach if reach < 60 else 8])):
             h[:, 0], h[:, 1] = 0.0, 1.0
             h[[f for f in flagged if 0 <= f < len(h)], 0] = 8.0
     hs = [rounded(h, dtype) for h in hs]
@@ -401,16 +404,18 @@ def test_latent_attention_part(dtype, shape, schedule, spiky):
     angle = np.float64 if dtype == torch.float32 else np.float32
     want = [M.latent_attention({"x." + k: v for k, v in w.items()}, "x.", m, h.astype(np.float64), np.arange(len(h)), eps,
                                store_of(dtype), angle) for h in hs]
-    harness = Harness([part.cache_spec()], dtype, page=page, pages=-(-150 // page) + -(-61 // page) + 2)
+    harness = Harness([part.cache_spec()], dtype, page=page, pages=-(-lengths[0] // page) + -(-61 // page) + 2)
     seqs = [harness.cache.create() for _ in lengths]
     fed = [0, 0]
     got = [np.zeros((n, hidden), np.float32) for n in lengths]
     if schedule == "portions":
-        steps = [(16, 1), (5, 9), (1, 1), (2, 3), (13, 8), (40, 2), (2, 30), (64, 2), (7, 5)]
+        steps = [(16, 1), (5, 9), (1, 1), (2, 3), (13, 8), (40, 2), (2, 30), (64, 2), (7, 5), (200, 1), (250, 1)]
     else:
-        steps = [(100, 20)] + [(1, 1)] * 50
+        steps = [(lengths[0] - 50, 20)] + [(1, 1)] * 50
     for step in steps:
         index = [i for i in range(2) if fed[i] < lengths[i]]
+        if not index:
+            break
         counts = [min(step[i], lengths[i] - fed[i]) for i in index]
         ctx, entries = harness.context([(seqs[i], [0] * n) for i, n in zip(index, counts)])
         h = torch.cat([dev(hs[i][fed[i]:fed[i] + n], dtype) for i, n in zip(index, counts)])
