@@ -6,7 +6,7 @@ namespace sprout {
 int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, const void* k_pool,
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
-                      int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale, int max_tile_ctx,
+                      int nq, int nkv, int hd, int page_size, int num_pages, ScoreStage st, float scale, int max_tile_ctx,
                       float* workspace, bool single);
 size_t attention_generic_workspace_floats(int dtype, int page_size, int n_tiles, int nq, int nkv, int hd, int max_tile_ctx,
                                           bool single);
@@ -20,13 +20,13 @@ int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_poo
                    const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
                    int max_decode_ctx, int max_tile_ctx, int mean_tile_walk, float* workspace, void* out, int nq, int nkv,
-                   int hd, int page_size, int num_pages, int window, float scale);
+                   int hd, int page_size, int num_pages, ScoreStage st, float scale);
 bool attention_decode_project_takes(int hd, int page_size, int nq, int nkv, int n_decode, int max_decode_ctx, int hidden);
 int attention_mfma_decode_project(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                                   const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                                   const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                                   float* workspace, const void* w_o, float* residual, int hidden, int nq, int nkv,
-                                  int hd, int page_size, int num_pages, int window, float scale);
+                                  int hd, int page_size, int num_pages, ScoreStage st, float scale);
 }  // namespace sprout
 
 using namespace sprout;
@@ -72,8 +72,10 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
                             const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
                             int64_t workspace_floats, void* out, int nq,
                             int nkv, int hd, int page_size, int num_pages, int window, float scale, int kernel_kind,
-                            int scores) {
-  SP_REQUIRE(scores == 0, "sp_attention: no kernel for score stage %d (0 = the scaled product alone)", scores);
+                            int scores, float softcap, const float* sinks, int mask_chunk) {
+  SP_REQUIRE(scores == 0 || (scores == 1 && softcap > 0.f), "sp_attention: no kernel for score stage %d (0 = the scaled product alone, 1 = capped by a positive number)", scores);
+  SP_REQUIRE(mask_chunk >= 0, "sp_attention: blocks of %d positions", mask_chunk);
+  const ScoreStage st = {window, mask_chunk, scores == 1 ? softcap : 0.f, sinks};
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_attention: unsupported dtype %d", dtype);
   SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "sp_attention: %d query heads do not divide into %d groups", nq, nkv);
   SP_REQUIRE(hd > 0 && hd <= 512, "sp_attention: head size %d is outside 1..512", hd);
@@ -96,7 +98,7 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
                "sp_attention: workspace of %lld floats is smaller than the %lld needed", (long long)workspace_floats,
                (long long)need);
     return attention_generic(s, dtype, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len,
-                             ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages, window, scale,
+                             ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages, st, scale,
                              max_tile_ctx, need ? workspace : nullptr, single);
   }
   if (plan[1]) {      // groups too large for the one-query kernel: the tile list holds every sequence, and that a step
@@ -114,7 +116,7 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
   return attention_mfma(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
                         n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx,
                         mean_tile_walk > 0 ? mean_tile_walk : max_tile_ctx, workspace, out,
-                        nq, nkv, hd, page_size, num_pages, window, scale);
+                        nq, nkv, hd, page_size, num_pages, st, scale);
 }
 
 // Whether sp_attention_decode_project takes a step of n_decode one-query sequences (bfloat16 only).
@@ -132,8 +134,11 @@ extern "C" int sp_attention_decode_project(void* stream, const void* q, int q_st
                                            const int32_t* q_start, const int32_t* ctx_len, const int32_t* decode_seqs,
                                            int n_decode, int max_decode_ctx, float* workspace, int64_t workspace_floats,
                                            const void* w_o, float* residual, int hidden, int nq, int nkv, int hd,
-                                           int page_size, int num_pages, int window, float scale, int scores) {
-  SP_REQUIRE(scores == 0, "sp_attention_decode_project: no kernel for score stage %d (0 = the scaled product alone)", scores);
+                                           int page_size, int num_pages, int window, float scale, int scores,
+                                           float softcap, const float* sinks, int mask_chunk) {
+  SP_REQUIRE(scores == 0 || (scores == 1 && softcap > 0.f), "sp_attention_decode_project: no kernel for score stage %d", scores);
+  SP_REQUIRE(mask_chunk >= 0, "sp_attention_decode_project: blocks of %d positions", mask_chunk);
+  const ScoreStage st = {window, mask_chunk, scores == 1 ? softcap : 0.f, sinks};
   SP_REQUIRE(sp_attention_decode_project_takes(hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden),
              "sp_attention_decode_project: hd=%d page=%d heads=%d/%d sequences=%d context=%d hidden=%d is not taken",
              hd, page_size, nq, nkv, n_decode, max_decode_ctx, hidden);
@@ -148,5 +153,5 @@ extern "C" int sp_attention_decode_project(void* stream, const void* q, int q_st
              (long long)workspace_floats, (long long)need);
   return attention_mfma_decode_project((hipStream_t)stream, q, q_stride, k_pool, v_pool, block_tables, max_blocks,
                                        q_start, ctx_len, decode_seqs, n_decode, max_decode_ctx, workspace, w_o, residual,
-                                       hidden, nq, nkv, hd, page_size, num_pages, window, scale);
+                                       hidden, nq, nkv, hd, page_size, num_pages, st, scale);
 }

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256) void attention_f32_decode_kernel(
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ tiles, float* __restrict__ out,
     float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits, int nq, int nkv, int page_size,
-    int num_pages, int window, float scale2) {
+    int num_pages, ScoreStage st, float scale2) {
   constexpr int HD = 16 * DT;
   extern __shared__ float f32_lds[];
   float* s_o = f32_lds;                                   // [4][16][HD + 1]
@@ -72,8 +72,10 @@ __global__ __launch_bounds__(256) void attention_f32_decode_kernel(
     s_table[threadIdx.x] = block_tables[size_t(seq) * max_blocks + min(table_first + int(threadIdx.x), max_blocks - 1)];
   const int q_row = q_start[seq];
   const int ctx = ctx_len[seq], pos = ctx - 1;
-  const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int k_lo = first_visible(pos, st.window, st.chunk);
   const int G = nq / nkv;
+  // capped scores: cap * tanh(s * scale / cap), in log2 units like everything the running softmax sees
+  const float cap2 = st.cap * kLog2e, per_cap = st.cap > 0.f ? scale2 / cap2 : 0.f;
   if (chunk0 > pos || chunk0 + kChunk <= k_lo) {
     // no visible key in this chunk: the merge reads every chunk's (maximum, sum), so an empty chunk says so itself
     if (n_splits > 1 && int(threadIdx.x) < G) {
@@ -99,6 +101,11 @@ __global__ __launch_bounds__(256) void attention_f32_decode_kernel(
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m = kNoKey, lsum = 0.f;
+  // a sink is a term of the denominator without a key: the first wave of the chunk that holds the query starts from it
+  if (st.sinks && wave == 0 && pos < chunk0 + kChunk && lr < G) {
+    m = st.sinks[g * G + lr] * kLog2e;
+    lsum = lj == 0 ? 1.f : 0.f;
+  }
   const int w0 = chunk0 + wave * kWaveKeys;
 
 #pragma unroll
@@ -140,7 +147,8 @@ __global__ __launch_bounds__(256) void attention_f32_decode_kernel(
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int key = key0 + 4 * lj + e;
-        sv[e] = (key >= k_lo && key <= pos) ? s[e] * scale2 : -INFINITY;
+        const float sc = st.cap > 0.f ? cap2 * tanhf(s[e] * per_cap) : s[e] * scale2;
+        sv[e] = (key >= k_lo && key <= pos) ? sc : -INFINITY;
         top = fmaxf(top, sv[e]);
       }
       top = max_over_quarters(top);
@@ -263,7 +271,7 @@ __global__ __launch_bounds__(64 * MAXW) void attention_f32_tiles_kernel(
     const float* __restrict__ q, int q_stride, const float* __restrict__ k_pool, const float* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ tiles,
-    float* __restrict__ out, int nq, int nkv, int page_size, int num_pages, int window, float scale2) {
+    float* __restrict__ out, int nq, int nkv, int page_size, int num_pages, ScoreStage st, float scale2) {
   constexpr int HD = 16 * DT;
   const int tile = gridDim.x - 1 - blockIdx.x;
   const int seq = tiles[2 * tile], q_off = tiles[2 * tile + 1];
@@ -298,12 +306,20 @@ __global__ __launch_bounds__(64 * MAXW) void attention_f32_tiles_kernel(
   }
   floatx4 o[2][DT];
   float m[2] = {kNoKey, kNoKey}, lsum[2] = {0.f, 0.f};
+  int qlo[2];        // the first key each of this lane's rows sees
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
+  for (int qt = 0; qt < 2; ++qt) {
+    qlo[qt] = first_visible(max(qpos[qt], 0), st.window, st.chunk);
+    if (st.sinks) {  // a term of the denominator without a key: the running softmax starts from it
+      m[qt] = st.sinks[head] * kLog2e;
+      lsum[qt] = lj == 0 ? 1.f : 0.f;
+    }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float cap2 = st.cap * kLog2e, per_cap = st.cap > 0.f ? scale2 / cap2 : 0.f;
 
-  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;     // the oldest key any query of the tile sees
+  const int k_lo = first_visible(pos0, st.window, st.chunk);       // the oldest key any query of the tile sees
   const int first_key = (k_lo / kStep) * kStep;
 
   auto load = [&](int key0, float4 (&kr)[DT], float4 (&vr)[DT]) {
@@ -331,12 +347,13 @@ __global__ __launch_bounds__(64 * MAXW) void attention_f32_tiles_kernel(
         s = mfma4(kr[c].z, qv[qt][c].z, s);
         s = mfma4(kr[c].w, qv[qt][c].w, s);
       }
-      const int hi = qpos[qt], lo = window > 0 ? max(0, hi - window + 1) : 0;
+      const int hi = qpos[qt], lo = qlo[qt];
       float sv[4], top = -INFINITY;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int key = key0 + 4 * lj + e;
-        sv[e] = (key >= lo && key <= hi) ? s[e] * scale2 : -INFINITY;      // hi = -1: a row that does not exist
+        const float sc = st.cap > 0.f ? cap2 * tanhf(s[e] * per_cap) : s[e] * scale2;
+        sv[e] = (key >= lo && key <= hi) ? sc : -INFINITY;      // hi = -1: a row that does not exist
         top = fmaxf(top, sv[e]);
       }
       top = max_over_quarters(top);
@@ -399,11 +416,11 @@ template <int DT>
 int launch_tiles(hipStream_t s, const float* q, int q_stride, const float* k_pool, const float* v_pool,
                  const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                  const int32_t* ctx_len, const int32_t* tiles, int n_tiles, float* out, int nq, int nkv, int page_size,
-                 int num_pages, int window, float scale) {
+                 int num_pages, ScoreStage st, float scale) {
   const int G = nq / nkv, parts = (G + 3) / 4;
   attention_f32_tiles_kernel<DT, (DT <= 8), 4><<<dim3(n_tiles, nkv * parts), 64 * min(G, 4), 0, s>>>(
       q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, out, nq, nkv, page_size,
-      num_pages, window, scale * kLog2e);
+      num_pages, st, scale * kLog2e);
   return check_launch("sp_attention (float32, tiles)");
 }
 
@@ -413,7 +430,7 @@ template <int DT, int SB>
 int launch_decode(hipStream_t s, const float* q, int q_stride, const float* k_pool, const float* v_pool,
                   const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* ctx_len,
                   const int32_t* tiles, int n_tiles, float* out, float* workspace, int n_splits, int nq, int nkv,
-                  int page_size, int num_pages, int window, float scale) {
+                  int page_size, int num_pages, ScoreStage st, float scale) {
   constexpr int HD = 16 * DT;
   const size_t lds = decode_lds_bytes(HD);
   static bool raised = false;
@@ -430,7 +447,7 @@ int launch_decode(hipStream_t s, const float* q, int q_stride, const float* k_po
   float* part_ml = workspace ? workspace + size_t(n_tiles) * nq * n_splits * HD : nullptr;
   attention_f32_decode_kernel<DT, SB><<<dim3(n_splits, nkv, n_tiles), 256, lds, s>>>(
       q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, ctx_len, tiles, out, part_o, part_ml, n_splits,
-      nq, nkv, page_size, num_pages, window, scale * kLog2e);
+      nq, nkv, page_size, num_pages, st, scale * kLog2e);
   if (check_launch("sp_attention (float32, one query)")) return 1;
   if (n_splits == 1) return 0;
   attention_f32_merge_kernel<<<dim3(n_tiles, nq), 64, 0, s>>>(part_o, part_ml, q_start, tiles, out, n_splits, nq, HD);
@@ -455,7 +472,7 @@ size_t attention_f32_decode_workspace_floats(int n_tiles, int nq, int hd, int ma
 int attention_f32_decode(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                          const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* ctx_len,
                          const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd, int page_size,
-                         int num_pages, int window, float scale, int max_ctx, float* workspace) {
+                         int num_pages, ScoreStage st, float scale, int max_ctx, float* workspace) {
   SP_REQUIRE(attention_f32_decode_takes(hd, page_size, nq, nkv), "sp_attention (float32, one query): sizes not taken");
   SP_REQUIRE(max_ctx <= max_blocks * page_size, "sp_attention: a context of %d tokens exceeds the block tables (%d pages of %d)",
              max_ctx, max_blocks, page_size);
@@ -467,7 +484,7 @@ int attention_f32_decode(hipStream_t s, const void* q, int q_stride, const void*
 #define SP_F32_DECODE(DT, SB)                                                                                     \
   return launch_decode<DT, SB>(s, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,          \
                                block_tables, max_blocks, q_start, ctx_len, tiles, n_tiles, (float*)out, workspace, \
-                               n_splits, nq, nkv, page_size, num_pages, window, scale)
+                               n_splits, nq, nkv, page_size, num_pages, st, scale)
   switch (hd / 16) {
     case 1: SP_F32_DECODE(1, 4);
     case 2: SP_F32_DECODE(2, 4);
@@ -492,7 +509,7 @@ int attention_f32_decode(hipStream_t s, const void* q, int q_stride, const void*
 int attention_f32_tiles(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                         const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                         const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd,
-                        int page_size, int num_pages, int window, float scale) {
+                        int page_size, int num_pages, ScoreStage st, float scale) {
   SP_REQUIRE(attention_f32_decode_takes(hd, page_size, nq, nkv), "sp_attention (float32, tiles): sizes not taken");
   SP_REQUIRE((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k_pool) | reinterpret_cast<uintptr_t>(v_pool) |
               reinterpret_cast<uintptr_t>(out)) % 16 == 0 && q_stride % 4 == 0,
@@ -501,14 +518,14 @@ int attention_f32_tiles(hipStream_t s, const void* q, int q_stride, const void* 
   case DT:                                                                                                        \
     return launch_tiles<DT>(s, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool, block_tables, \
                             max_blocks, q_start, q_len, ctx_len, tiles, n_tiles, (float*)out, nq, nkv, page_size,  \
-                            num_pages, window, scale)
+                            num_pages, st, scale)
   switch (hd / 16) {
     SP_F32_TILES(1); SP_F32_TILES(2); SP_F32_TILES(3); SP_F32_TILES(4); SP_F32_TILES(5); SP_F32_TILES(6);
     SP_F32_TILES(7); SP_F32_TILES(8); SP_F32_TILES(9); SP_F32_TILES(10); SP_F32_TILES(11); SP_F32_TILES(12);
     SP_F32_TILES(13); SP_F32_TILES(14); SP_F32_TILES(15);
     default: return launch_tiles<16>(s, (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,
                                      block_tables, max_blocks, q_start, q_len, ctx_len, tiles, n_tiles, (float*)out, nq,
-                                     nkv, page_size, num_pages, window, scale);
+                                     nkv, page_size, num_pages, st, scale);
   }
 #undef SP_F32_TILES
 }

@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ tiles,
-    T* __restrict__ out, int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale,
+    T* __restrict__ out, int nq, int nkv, int hd, int page_size, int num_pages, ScoreStage st, float scale,
     float* __restrict__ part, int chunk) {
   extern __shared__ float lds[];
   // rows one float longer than their content: the four query rows that a wave reads at the same column
@@ -115,13 +115,16 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   src.nkv = nkv; src.g = GROUPED ? blockIdx.y : blockIdx.y / G; src.hd = hd; src.page_size = page_size; src.num_pages = num_pages; src.max_blocks = max_blocks;
   // one past the last visible key of the tile (GROUPED: its rows are heads of one query, at pos0)
   src.k_end = pos0 + (GROUPED ? 1 : nvalid);
-  src.k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  src.k_lo = first_visible(pos0, st.window, st.chunk);        // the oldest key any row of the tile sees
+  const int my_lo = first_visible(my_pos, st.window, st.chunk);
   const int n_chunks = gridDim.z, first_key = blockIdx.z * chunk;   // this block's keys: first_key .. + chunk - 1
   if (blockIdx.z + 1 < n_chunks) src.k_end = min(src.k_end, first_key + chunk);   // the last chunk: all that is left
   src.by_hd.set(hd);
   src.by_page.set(page_size);
   const int k_lo = src.k_lo, k_end = src.k_end;
   float m = -INFINITY, l = 0.f;
+  // a sink is a term of the denominator without a key: the block of the first chunk starts from it
+  if (st.sinks && blockIdx.z == 0) { m = st.sinks[h]; l = 1.f; }
   float acc[MAXD];
 #pragma unroll
   for (int i = 0; i < MAXD; ++i) acc[i] = 0.f;
@@ -146,8 +149,10 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       float dot = 0.f;
 #pragma unroll 8   // several LDS reads on their way at a time; the order of the sum stays
       for (int d = 0; d < hd; ++d) dot = fmaf(Qs[r * kv_stride + d], KVs[c * kv_stride + d], dot);
-      const bool visible = r < nvalid && j >= k_lo && j <= my_pos && (window <= 0 || my_pos - j < window);
-      s[u] = visible ? dot * scale : -INFINITY;
+      const bool visible = r < nvalid && j >= my_lo && j <= my_pos;
+      dot *= scale;
+      if (st.cap > 0.f) dot = st.cap * tanhf(dot / st.cap);
+      s[u] = visible ? dot : -INFINITY;
       row_max = fmaxf(row_max, s[u]);
     }
 #pragma unroll
@@ -245,12 +250,12 @@ size_t attention_f32_decode_workspace_floats(int n_tiles, int nq, int hd, int ma
 int attention_f32_decode(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                          const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* ctx_len,
                          const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd, int page_size,
-                         int num_pages, int window, float scale, int max_ctx, float* workspace);
+                         int num_pages, ScoreStage st, float scale, int max_ctx, float* workspace);
 
 int attention_f32_tiles(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                         const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                         const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out, int nq, int nkv, int hd,
-                        int page_size, int num_pages, int window, float scale);
+                        int page_size, int num_pages, ScoreStage st, float scale);
 
 // Float32 storage goes to the matrix-core kernels of attention_f32.hip where they take the sizes: a step of
 // one-query sequences to the one that shares a sequence's keys out over blocks, any other to the one that walks
@@ -293,7 +298,7 @@ template <typename T>
 int launch_attention_generic(hipStream_t s, const void* q, int q_stride, const void* k_pool, const void* v_pool,
                              const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                              const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles,
-                             void* out, int nq, int nkv, int hd, int page_size, int num_pages, int window,
+                             void* out, int nq, int nkv, int hd, int page_size, int num_pages, ScoreStage st,
                              float scale, int max_tile_ctx, float* workspace, bool single) {
   const size_t lds = sizeof(float) * (size_t(AQ + AK) * (hd + 1) + AQ * (AK + 1));
   const bool grouped = generic_grouped(single, nq, nkv);
@@ -305,11 +310,11 @@ int launch_attention_generic(hipStream_t s, const void* q, int q_stride, const v
   if (grouped)                                                                                                 \
     attention_generic_kernel<T, MAXD, true><<<grid, 256, lds, s>>>(                                            \
         (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, block_tables, max_blocks, q_start, q_len,  \
-        ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale, workspace, chunk);         \
+        ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, st, scale, workspace, chunk);             \
   else                                                                                                         \
     attention_generic_kernel<T, MAXD, false><<<grid, 256, lds, s>>>(                                           \
         (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, block_tables, max_blocks, q_start, q_len,  \
-        ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, window, scale, workspace, chunk)
+        ctx_len, tiles, (T*)out, nq, nkv, hd, page_size, num_pages, st, scale, workspace, chunk)
   if (hd <= 64) { SP_ATT(4); }
   else if (hd <= 128) { SP_ATT(8); }
   else if (hd <= 256) { SP_ATT(16); }
@@ -341,24 +346,24 @@ int launch_attention_generic(hipStream_t s, const void* q, int q_stride, const v
 int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, const void* k_pool,
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
-                      int nq, int nkv, int hd, int page_size, int num_pages, int window, float scale, int max_tile_ctx,
+                      int nq, int nkv, int hd, int page_size, int num_pages, ScoreStage st, float scale, int max_tile_ctx,
                       float* workspace, bool single) {
   SP_REQUIRE(int64_t(max_blocks) * page_size < (int64_t(1) << 24),
              "sp_attention: block tables of %d pages of %d tokens exceed the 2^24 positions this kernel counts",
              max_blocks, page_size);
   if (f32_one_query(dtype, single, nq, nkv, hd, page_size))
     return attention_f32_decode(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, ctx_len, tiles, n_tiles,
-                                out, nq, nkv, hd, page_size, num_pages, window, scale, max_tile_ctx, workspace);
+                                out, nq, nkv, hd, page_size, num_pages, st, scale, max_tile_ctx, workspace);
   if (attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size))
     return attention_f32_tiles(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
-                               n_tiles, out, nq, nkv, hd, page_size, num_pages, window, scale);
+                               n_tiles, out, nq, nkv, hd, page_size, num_pages, st, scale);
   if (dtype == kF32)
     return launch_attention_generic<float>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                            q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size,
-                                           num_pages, window, scale, max_tile_ctx, workspace, single);
+                                           num_pages, st, scale, max_tile_ctx, workspace, single);
   return launch_attention_generic<bf16_t>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start,
                                           q_len, ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages,
-                                          window, scale, max_tile_ctx, workspace, single);
+                                          st, scale, max_tile_ctx, workspace, single);
 }
 
 }  // namespace sprout

@@ -114,11 +114,33 @@ __device__ __forceinline__ float max_over_quarters(float x) {
 // starts at kNoKeyYet.
 // CONTIG: the step's keys in the order 8 lj + 4 kt + r (a lane's eight keys in a row, as the staged kernel reads its
 // values from LDS in one piece) instead of 16 kt + 4 lj + r; whoever loads the step lays its key rows out to match.
+// What a step needs of the score stage: whether rows differ in the first key they see (a window or blocks of
+// positions: every step is masked then), and the two factors of a capped score, taken on the raw product so that
+// what follows multiplies by scale2 as ever: s <- cap_mul * tanh(s * cap_arg), cap_arg = scale / cap, cap_mul = cap / scale.
+struct StepRule {
+  bool rows_differ;
+  float cap_arg, cap_mul;
+};
+__device__ __forceinline__ StepRule step_rule(const ScoreStage& st, float scale2) {
+  StepRule rule;
+  rule.rows_differ = st.window > 0 || st.chunk > 0;
+  const float scale = scale2 / kLog2e;
+  rule.cap_arg = st.cap > 0.f ? scale / st.cap : 0.f;
+  rule.cap_mul = st.cap > 0.f ? st.cap / scale : 0.f;
+  return rule;
+}
+// tanh(x) = 1 - 2 / (exp(2x) + 1): exact to a few units of the last place of 1, which a capped score of the
+// bfloat16 path does not see; the ends come out as -1 and 1.
+__device__ __forceinline__ float fast_tanh(float x) {
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x * (2.0f * kLog2e)) + 1.0f);
+}
+
+// qlo[qt]: the first key that this lane's row sees (first_visible of its position).
 template <int DT, int NQT, bool MASKED, bool LAZY, bool CONTIG>
 __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
                                                  floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT],
-                                                 int key0, int k_lo, const int (&qpos)[NQT], int window,
-                                                 float scale2) {
+                                                 int key0, int k_lo, const int (&qpos)[NQT], const int (&qlo)[NQT],
+                                                 const StepRule& rule, float scale2) {
   constexpr int HC = (DT + 1) / 2;
   const int lane = threadIdx.x & 63, lj = lane >> 4;
 
@@ -131,6 +153,14 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
 #pragma unroll
       for (int c = 0; c < HC; ++c) s[qt][kt] = mfma16(r.ka[kt][c], qop[qt][c], s[qt][kt]);
     }
+  if (rule.cap_mul > 0.f) {      // the same in every lane
+#pragma unroll
+    for (int qt = 0; qt < NQT; ++qt)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) s[qt][kt][r4] = rule.cap_mul * fast_tanh(s[qt][kt][r4] * rule.cap_arg);
+  }
 
   float raw[NQT];
   bool grown = false;
@@ -139,7 +169,7 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
     if (MASKED) {
       // visible keys of this lane's row: lo .. lo + span (none when span < 0), tested with one unsigned compare
       const int hi = qpos[qt];
-      const int lo = window > 0 ? max(k_lo, hi - window + 1) : k_lo;
+      const int lo = max(k_lo, qlo[qt]);
       const int span = hi - lo;
       const unsigned limit = span >= 0 ? unsigned(span) : 0u;
       const int base = span >= 0 ? lo : key0 + 64;          // key - base < 0 for every key of the step: none passes
@@ -198,16 +228,16 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
 }
 
 // `first_pos`: smallest position among the rows that exist; a step whose 32 keys all lie at or before
-// it (and inside [k_lo, ...) with no window) needs no masking.
+// it (and inside [k_lo, ...) where all rows see the same first key) needs no masking.
 template <int DT, int NQT, bool LAZY = true, bool CONTIG = false>
 __device__ __forceinline__ void attend_step(const KVStep<DT>& r, const bf16x8 (&qop)[NQT][(DT + 1) / 2],
                                             floatx4 (&o)[NQT][DT], float (&m)[NQT], float (&lsum)[NQT], int key0,
-                                            int k_lo, const int (&qpos)[NQT], int window, float scale2,
-                                            int first_pos) {
-  if (window <= 0 && key0 >= k_lo && key0 + 31 <= first_pos)
-    attend_step_impl<DT, NQT, false, LAZY, CONTIG>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+                                            int k_lo, const int (&qpos)[NQT], const int (&qlo)[NQT],
+                                            const StepRule& rule, float scale2, int first_pos) {
+  if (!rule.rows_differ && key0 >= k_lo && key0 + 31 <= first_pos)
+    attend_step_impl<DT, NQT, false, LAZY, CONTIG>(r, qop, o, m, lsum, key0, k_lo, qpos, qlo, rule, scale2);
   else
-    attend_step_impl<DT, NQT, true, LAZY, CONTIG>(r, qop, o, m, lsum, key0, k_lo, qpos, window, scale2);
+    attend_step_impl<DT, NQT, true, LAZY, CONTIG>(r, qop, o, m, lsum, key0, k_lo, qpos, qlo, rule, scale2);
 }
 
 template <int DT>
@@ -228,7 +258,7 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, int nq, int nkv, int page_size, int num_pages,
-    int window, float scale2) {
+    ScoreStage st, float scale2) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   const int seq = tiles[2 * blockIdx.x], q_off = tiles[2 * blockIdx.x + 1];
   const int h = blockIdx.y, g = h / (nq / nkv);
@@ -247,7 +277,7 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
   kv.table = block_tables + size_t(seq) * max_blocks;
 
   bf16x8 qop[NQT][HC];
-  int qpos[NQT];
+  int qpos[NQT], qlo[NQT];
   floatx4 o[NQT][DT];
   float m[NQT], lsum[NQT];
 #pragma unroll
@@ -255,15 +285,18 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
     const int row = 16 * qt + lr;
     const bool valid = row < nvalid;
     qpos[qt] = valid ? pos0 + row : -1;
+    qlo[qt] = first_visible(max(qpos[qt], 0), st.window, st.chunk);
     load_q_operand<DT>(qop[qt], valid ? q + size_t(qs + q_off + row) * q_stride + h * HD : nullptr);
-    m[qt] = kNoKeyYet;
-    lsum[qt] = 0.f;
+    // a sink is a term of the denominator without a key: the running softmax starts from it (one lane of a row's four)
+    m[qt] = st.sinks ? st.sinks[h] * kLog2e : kNoKeyYet;
+    lsum[qt] = st.sinks && lj == 0 ? 1.f : 0.f;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
   const int k_hi = pos0 + nvalid - 1;
-  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int k_lo = first_visible(pos0, st.window, st.chunk);
+  const StepRule rule = step_rule(st, scale2);
   // the next step's keys and values are on their way while the current step is multiplied
   KVStep<DT> cur, nxt;
   int key0 = (k_lo >> 5) << 5;
@@ -271,7 +304,7 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
   for (; key0 <= k_hi; key0 += 32) {
     const bool more = key0 + 32 <= k_hi;
     if (more) load_step<DT>(nxt, kv, key0 + 32, k_lo, k_hi);
-    attend_step<DT, NQT>(cur, qop, o, m, lsum, key0, k_lo, qpos, window, scale2, pos0);
+    attend_step<DT, NQT>(cur, qop, o, m, lsum, key0, k_lo, qpos, qlo, rule, scale2, pos0);
     if (more) cur = nxt;
   }
 
@@ -314,7 +347,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ q_len, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ tiles, uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int n_splits, int stages_per_split, int nq, int nkv, int page_shift, int num_pages,
-    int window, float scale2, int n_tiles) {
+    ScoreStage st, float scale2, int n_tiles) {
   constexpr int HD = 16 * DT, HC = (DT + 1) / 2;
   constexpr int THREADS = 64 * WPT * HPB;
   constexpr int WAVE_KEYS = kStageKeys / WPT;          // keys of a stage that one wave of a team takes
@@ -358,7 +391,8 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   if (nvalid <= 0) continue;
   const int pos0 = ctx - qlen + q_off;
   const int k_hi = pos0 + nvalid - 1;
-  const int k_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int k_lo = first_visible(pos0, st.window, st.chunk);
+  const StepRule rule = step_rule(st, scale2);
 
   const int32_t* table = block_tables + size_t(seq) * max_blocks;
   const int first_page = k_lo >> page_shift, n_pages = (k_hi >> page_shift) - first_page + 1;
@@ -378,7 +412,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   const uint16_t* vbase = v_pool + (size_t(g) << page_shift) * HD;
 
   bf16x8 qop[NQT][HC];
-  int qpos[NQT];
+  int qpos[NQT], qlo[NQT];
   floatx4 o[NQT][DT];
   float m[NQT], lsum[NQT];
 #pragma unroll
@@ -386,9 +420,13 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
     const int row = 16 * qt + lr;
     const bool valid = row < nvalid;
     qpos[qt] = valid ? pos0 + row : -1;
+    qlo[qt] = first_visible(max(qpos[qt], 0), st.window, st.chunk);
     load_q_operand<DT>(qop[qt], valid ? q + size_t(qs + q_off + row) * q_stride + h * HD : nullptr);
-    m[qt] = kNoKeyYet;
-    lsum[qt] = 0.f;
+    // a sink is a term of the denominator without a key: one wave of the team, in the block of the first split,
+    // starts its running softmax from it (one lane of a row's four)
+    const bool with_sink = st.sinks && wave == 0 && blockIdx.z == 0;
+    m[qt] = with_sink ? st.sinks[h] * kLog2e : kNoKeyYet;
+    lsum[qt] = with_sink && lj == 0 ? 1.f : 0.f;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
@@ -499,7 +537,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
         }
         // (the unpaired block of 16 waves has no register to spare: the lazy form made it spill 36 instead of 2,
         // 529 -> 690 us for 2,048 queries over 32,768 keys; the paired one gained with it, 290 -> 264 us at 8,192)
-        attend_step<DT, NQT, !(HPB * WPT == 16 && !PAIRED), true>(r, qop, o, m, lsum, wkey, k_lo, qpos, window, scale2, pos0);
+        attend_step<DT, NQT, !(HPB * WPT == 16 && !PAIRED), true>(r, qop, o, m, lsum, wkey, k_lo, qpos, qlo, rule, scale2, pos0);
       }
     }
   };
@@ -611,7 +649,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     const uint16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ decode_seqs,
     uint16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits, int nq,
-    int nkv, int kv_stored, int page_size, int num_pages, int window, float scale2) {
+    int nkv, int kv_stored, int page_size, int num_pages, ScoreStage st, float scale2) {
   // nkv: the sets of query heads that a block takes at once (blockIdx.y); kv_stored: the key/value heads the pools
   // hold.  They are the same unless a key/value head serves more query heads than the 16 rows of a block: then
   // its heads are taken in nkv / kv_stored sets that read the same keys.
@@ -633,7 +671,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   // without a list, sequence i's one query is row i
   const int q_row = decode_seqs ? q_start[seq] : seq;
   const int ctx = ctx_len[seq], pos = ctx - 1;
-  const int k_lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int k_lo = first_visible(pos, st.window, st.chunk);
   const int G = nq / nkv;
   if (chunk0 > pos || chunk0 + kDecodeChunk <= k_lo) {
     // no visible key in this chunk: the merge kernel reads every chunk's (maximum, sum) without looking at
@@ -659,11 +697,18 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   kv.page_shift = page_shift;
 
   bf16x8 qop[1][HC];
-  int qpos[1] = {lr < G ? pos : -1};
+  int qpos[1] = {lr < G ? pos : -1}, qlo[1] = {k_lo};
+  const StepRule rule = step_rule(st, scale2);
   load_q_operand<DT>(qop[0], lr < G ? q + size_t(q_row) * q_stride + (g * G + lr) * HD : nullptr);
   __syncthreads();   // the page numbers are in LDS
   floatx4 o[1][DT];
   float m[1] = {kNoKeyYet}, lsum[1] = {0.f};
+  // a sink is a term of the denominator without a key: the first wave of the chunk that holds the query (a chunk
+  // that always runs) starts its running softmax from it, one lane of a row's four
+  if (st.sinks && wave == 0 && pos < chunk0 + kDecodeChunk && lr < G) {
+    m[0] = st.sinks[g * G + lr] * kLog2e;
+    lsum[0] = lj == 0 ? 1.f : 0.f;
+  }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[0][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
 
@@ -679,7 +724,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   }
 #pragma unroll
   for (int i = 0; i < kDecodeWaveKeys / 32; ++i)
-    if (live[i]) attend_step<DT, 1>(steps[i], qop, o, m, lsum, w0 + 32 * i, k_lo, qpos, window, scale2, pos);
+    if (live[i]) attend_step<DT, 1>(steps[i], qop, o, m, lsum, w0 + 32 * i, k_lo, qpos, qlo, rule, scale2, pos);
   float l = lsum[0];
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -987,7 +1032,7 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
                        const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                        const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs,
                        int n_decode, int max_decode_ctx, int max_tile_ctx, int mean_tile_walk, float* workspace,
-                       void* out, int nq, int nkv, int page_size, int num_pages, int window, float scale) {
+                       void* out, int nq, int nkv, int page_size, int num_pages, ScoreStage st, float scale) {
   constexpr int HD = 16 * DT;
   constexpr int NQT = 2;
   const float scale2 = scale * kLog2e;
@@ -1009,7 +1054,7 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
 #define SP_STAGED(HPB, WPT, AHEAD, PAIRED)                                                                      \
   attention_prefill_staged_kernel<DT, NQT, HPB, WPT, AHEAD, PAIRED><<<grid, 64 * WPT * HPB, 0, s>>>(            \
       qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, part_o,   \
-      part_ml, splits, per_split, nq, nkv, page_shift, num_pages, window, scale2, n_tiles)
+      part_ml, splits, per_split, nq, nkv, page_shift, num_pages, st, scale2, n_tiles)
       // the same cases as staged_shape() and staged_paired()
       if (paired) {
         if (shape.hpb == 1) SP_STAGED(1, 4, false, true);
@@ -1028,7 +1073,7 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
     } else {
       attention_prefill_kernel<DT, NQT><<<dim3(n_tiles, nq), 64, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, q_len, ctx_len, tiles, (uint16_t*)out, nq, nkv,
-          page_size, num_pages, window, scale2);
+          page_size, num_pages, st, scale2);
     }
     if (check_launch("sp_attention (prefill)")) return 1;
   }
@@ -1039,11 +1084,11 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
     if ((page_size & (page_size - 1)) == 0)
       attention_decode_kernel<DT, true><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
-          n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window, scale2);
+          n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, st, scale2);
     else
       attention_decode_kernel<DT, false><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
           qp, q_stride, kp, vp, block_tables, max_blocks, q_start, ctx_len, decode_seqs, (uint16_t*)out, part_o, part_ml,
-          n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window, scale2);
+          n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, st, scale2);
     if (check_launch("sp_attention (decode)")) return 1;
     if (n_splits > 1) {
       if (n_splits <= 16)
@@ -1062,12 +1107,12 @@ int attention_mfma(hipStream_t s, const void* q, int q_stride, const void* k_poo
                    const int32_t* block_tables, int max_blocks, const int32_t* q_start, const int32_t* q_len,
                    const int32_t* ctx_len, const int32_t* tiles, int n_tiles, const int32_t* decode_seqs, int n_decode,
                    int max_decode_ctx, int max_tile_ctx, int mean_tile_walk, float* workspace, void* out, int nq, int nkv,
-                   int hd, int page_size, int num_pages, int window, float scale) {
+                   int hd, int page_size, int num_pages, ScoreStage st, float scale) {
 #define SP_MFMA(DT)                                                                                              \
   case DT:                                                                                                       \
     return launch_mfma<DT>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len,    \
                            tiles, n_tiles, decode_seqs, n_decode, max_decode_ctx, max_tile_ctx, mean_tile_walk,  \
-                           workspace, out, nq, nkv, page_size, num_pages, window, scale)
+                           workspace, out, nq, nkv, page_size, num_pages, st, scale)
   switch (hd / 16) {
     SP_MFMA(1); SP_MFMA(2); SP_MFMA(3); SP_MFMA(4); SP_MFMA(5); SP_MFMA(6); SP_MFMA(8);
   }
@@ -1105,7 +1150,7 @@ static int launch_decode_project(hipStream_t s, const void* q, int q_stride, con
                                  const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                                  const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                                  float* workspace, const void* w_o, float* residual, int hidden, int nq, int nkv,
-                                 int page_size, int num_pages, int window, float scale) {
+                                 int page_size, int num_pages, ScoreStage st, float scale) {
   constexpr int HD = 16 * DT;
   const int n_splits = (max_decode_ctx + kDecodeChunk - 1) / kDecodeChunk;
   float* part_o = workspace;
@@ -1113,12 +1158,12 @@ static int launch_decode_project(hipStream_t s, const void* q, int q_stride, con
   if ((page_size & (page_size - 1)) == 0)
     attention_decode_kernel<DT, true><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
         (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
-        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window,
+        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, st,
         scale * kLog2e);
   else
     attention_decode_kernel<DT, false><<<dim3(n_splits, decode_sets(nq, nkv), n_decode), 256, 0, s>>>(
         (const uint16_t*)q, q_stride, (const uint16_t*)k_pool, (const uint16_t*)v_pool, block_tables, max_blocks, q_start,
-        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, window,
+        ctx_len, decode_seqs, nullptr, part_o, part_ml, n_splits, nq, decode_sets(nq, nkv), nkv, page_size, num_pages, st,
         scale * kLog2e);
   if (check_launch("sp_attention_decode_project (decode)")) return 1;
   const int tpw = project_tiles_per_wave(n_decode, nq, hidden);
@@ -1138,12 +1183,12 @@ int attention_mfma_decode_project(hipStream_t s, const void* q, int q_stride, co
                                   const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                                   const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                                   float* workspace, const void* w_o, float* residual, int hidden, int nq, int nkv,
-                                  int hd, int page_size, int num_pages, int window, float scale) {
+                                  int hd, int page_size, int num_pages, ScoreStage st, float scale) {
 #define SP_MFMA(DT)                                                                                              \
   case DT:                                                                                                       \
     return launch_decode_project<DT>(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, ctx_len, \
                                      decode_seqs, n_decode, max_decode_ctx, workspace, w_o, residual, hidden,    \
-                                     nq, nkv, page_size, num_pages, window, scale)
+                                     nq, nkv, page_size, num_pages, st, scale)
   switch (hd / 16) {
     SP_MFMA(1); SP_MFMA(2); SP_MFMA(3); SP_MFMA(4); SP_MFMA(5); SP_MFMA(6); SP_MFMA(8);
   }

@@ -45,6 +45,33 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return total;
 }
 
+// Activations of a gated product, numbered as in the C interface: 0 = SiLU(g) * u; 1 = the clamped form
+// g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1).
+enum GateAct : int { kActSilu = 0, kActClampedSwish = 1, kGateActs = 2 };
+constexpr float kSwishSlope = 1.702f;
+__device__ __forceinline__ float gated_value(float g, float u, int act, float limit) {
+  if (act == kActClampedSwish) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-kSwishSlope * g)) * (u + 1.0f);
+  }
+  return g / (1.0f + expf(-g)) * u;
+}
+
+// Which earlier keys a query sees, and what stands between q . k and the softmax.
+struct ScoreStage {
+  int window;          // > 0: keys with position - key < window
+  int chunk;           // > 0: only keys of the query's own block of `chunk` positions, counted from position 0
+  float cap;           // > 0: the scaled score s becomes cap * tanh(s / cap)
+  const float* sinks;  // one number per query head whose exponential joins the softmax's denominator (null: none)
+};
+// The first key that a query at `pos` sees.
+__device__ __forceinline__ int first_visible(int pos, int window, int chunk) {
+  int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, pos - pos % chunk);
+  return lo;
+}
+
 // Error text of the last failed call on this thread.
 void set_error(const char* fmt, ...);
 int check_launch(const char* what);

@@ -80,15 +80,18 @@ __global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const int32_t* 
 }
 
 // ---------------------------------------------------------------- SiLU(gate) * up
+// row_gate (may be null): the token's row is also multiplied by sigmoid(row_gate[t * row_gate_stride]), float32.
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I) {
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, int act, float limit,
+                                const float* __restrict__ row_gate, long long row_gate_stride) {
   const int t = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= I) return;
   const float g = to_float(gu[size_t(t) * 2 * I + i]);
   const float u = to_float(gu[size_t(t) * 2 * I + I + i]);
-  const float s = g / (1.0f + expf(-g));
-  out[size_t(t) * I + i] = from_float<T>(s * u);
+  float v = gated_value(g, u, act, limit);
+  if (row_gate) v *= 1.0f / (1.0f + expf(-row_gate[size_t(t) * row_gate_stride]));
+  out[size_t(t) * I + i] = from_float<T>(v);
 }
 
 // ---------------------------------------------------------------- rotation + cache write
@@ -279,14 +282,15 @@ extern "C" int sp_rmsnorm(void* stream, const float* x, const int32_t* rows, int
   return check_launch("sp_rmsnorm");
 }
 
-extern "C" int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation) {
-  SP_REQUIRE(activation == 0, "sp_silu_mul: no kernel for activation %d (0 = SiLU)", activation);
+extern "C" int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation, float limit,
+                           const float* row_gate, long long row_gate_stride) {
+  SP_REQUIRE(activation >= 0 && activation < kGateActs, "sp_silu_mul: no kernel for activation %d", activation);
   SP_REQUIRE(T >= 0 && I > 0, "sp_silu_mul: bad sizes T=%d I=%d", T, I);
   if (T == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((I + 255) / 256, T);
-  if (dtype == kF32) silu_mul_kernel<float><<<grid, 256, 0, s>>>((const float*)gu, (float*)out, I);
-  else if (dtype == kBF16) silu_mul_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, I);
+  if (dtype == kF32) silu_mul_kernel<float><<<grid, 256, 0, s>>>((const float*)gu, (float*)out, I, activation, limit, row_gate, row_gate_stride);
+  else if (dtype == kBF16) silu_mul_kernel<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)gu, (bf16_t*)out, I, activation, limit, row_gate, row_gate_stride);
   else SP_REQUIRE(false, "sp_silu_mul: unsupported dtype %d", dtype);
   return check_launch("sp_silu_mul");
 }

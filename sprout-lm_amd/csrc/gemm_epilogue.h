@@ -17,6 +17,9 @@ struct RopeArgs {
   uint16_t* v_pool;              // [page][kv head][dim][slot]
   int nq, nkv, hd, page_size;
   const float2* table;           // [T][hd / 2] (cosine, sine) of positions[t] * inv_freq[d], or null: computed here
+  // the gated epilogue (kSilu) reads only these: which activation (GateAct of common.h; 0 = SiLU) and its limit
+  int act;
+  float limit;
 };
 
 // Orders a wave's LDS writes before its own later reads of what other lanes wrote (and the reverse).
@@ -124,7 +127,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[WM][WN], float* tu
           for (int r = 0; r < 4; ++r) {
             const float g = to_float(bf16_t{f32_to_bf16_bits(acc[i][2 * m][4 * rg + r])});
             const float u = to_float(bf16_t{f32_to_bf16_bits(acc[i][(2 * m + 1) % WN][4 * rg + r])});
-            v[r] = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
+            v[r] = rope.act == kActSilu ? g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u : gated_value(g, u, rope.act, rope.limit);
           }
           uint16_t* dst = reinterpret_cast<uint16_t*>(out) + size_t(t) * N + n;
           if (n + 4 <= N && (N & 3) == 0) *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));

@@ -52,6 +52,9 @@ struct FusedArgs {
   uint16_t* v_pool;
   int nq, nkv, hd, page_size, rotary_dim;
   int page_shift;            // page_size == 1 << page_shift, or -1 where it is no power of two
+  // kEpiSilu: which gated activation (GateAct of common.h) and its limit
+  int act;
+  float limit;
 };
 
 // A bias value as it lies in memory (bfloat16 bits or float32 bits), and its value.  The two are kept apart
@@ -400,7 +403,7 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         const float gv = summed(gate >> 4, gate & 15, tn), uv = summed(up >> 4, up & 15, tn);
         // the engine keeps gate and up as bfloat16 before the gated product; keep the same roundings
         const float g = to_float(bf16_t{f32_to_bf16_bits(gv)}), u = to_float(bf16_t{f32_to_bf16_bits(uv)});
-        reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(g / (1.0f + expf(-g)) * u);
+        reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(gated_value(g, u, a.act, a.limit));
       }
       continue;
     }
@@ -584,7 +587,7 @@ extern "C" int sp_gemm_decode(void* stream, const void* x, const float* residual
                               int N, int K);
 
 namespace sprout {
-int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K);
+int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit);
 bool gemm_pipe_takes(int T, int N, int K);
 bool gemm_pipe_rope_takes(int T, int N, int K, int hd);
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
@@ -593,8 +596,9 @@ int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dt
 }
 
 extern "C" int sp_fused_supported(int kind, int T, int N, int K, int hd, int rotary_dim, int norm, int variant) {
-  if (variant != 0) return 0;   // the one pairing (halves) and the one activation (SiLU) these kernels have
-  if (kind == kEpiSilu && T > 64) return !norm && K % 8 == 0 && N % 2 == 0;   // the tiled kernel's gated epilogue
+  if (kind == kEpiSilu ? (variant < 0 || variant >= kGateActs) : variant != 0) return 0;   // the one pairing (halves); the gate activations of common.h
+  // the tiled kernel's gated epilogue (its pipelined form has every activation, the older tiles SiLU alone)
+  if (kind == kEpiSilu && T > 64) return !norm && K % 8 == 0 && N % 2 == 0 && (variant == 0 || gemm_pipe_takes(T, N, K));
   if (kind == kEpiRope && T > 64) return !norm && rotary_dim == hd && gemm_pipe_rope_takes(T, N, K, hd);   // and its rotating one
   if (!fused_shape_ok(T, K, norm != 0)) return 0;
   if (kind == kEpiRope) return hd % 16 == 0 && (rotary_dim == hd || rotary_dim == 0) && N % hd == 0;
@@ -688,8 +692,8 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
 // out[T, I] = silu(x . w_gate^T) * (x . w_up^T) with w = [gate rows; up rows] of [2 I, K].
 extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype,
                                const void* norm_w, float eps, const void* w, void* out, int T, int I, int K,
-                               int activation) {
-  SP_REQUIRE(activation == 0, "sp_gate_up_silu: no kernel for activation %d (0 = SiLU)", activation);
+                               int activation, float limit) {
+  SP_REQUIRE(activation >= 0 && activation < kGateActs, "sp_gate_up_silu: no kernel for activation %d", activation);
   SP_REQUIRE(sp_fused_supported(kEpiSilu, T, 2 * I, K, 0, 0, residual != nullptr, activation),
              "sp_gate_up_silu: shape T=%d I=%d K=%d is not taken", T, I, K);
   SP_REQUIRE((x || residual) && w && out, "sp_gate_up_silu: null operand");
@@ -701,11 +705,12 @@ extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residua
   const size_t weights = size_t(2) * I * K;
   const int fused_up_to = weights >= (size_t(200) << 20) ? 4 : weights >= (size_t(64) << 20) ? 8 : 16;
   if (T > 64 || (T > fused_up_to && !residual && gemm_pipe_takes(T, 2 * I, K)))
-    return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K);
+    return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K, activation, limit);
   FusedArgs a = {};
   a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
   a.w = (const uint16_t*)w; a.out = out;
   a.T = T; a.N = 2 * I; a.K = K; a.k_per_split = (K + 63) / 64 * 64; a.partner = I;
+  a.act = activation; a.limit = limit;
   a.rows_per_block = silu_rows_per_block(T, I, K, residual != nullptr);
   return fused_norm<kEpiSilu>((hipStream_t)stream, a, residual != nullptr, (I + a.rows_per_block - 1) / a.rows_per_block, 1);
 }

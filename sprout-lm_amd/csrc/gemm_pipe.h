@@ -273,7 +273,7 @@ inline int launch_pipe_mode(hipStream_t s, int splits, const TE* x, const TE* w,
 // The grouped form over `max_tiles` tiles of at most BM rows (see PipeGroups); K a multiple of 64, no split of K.
 template <int WM, int WN, int WAVES_M, int WAVES_N, int STAGES, int MODE>
 inline int launch_pipe_grouped(hipStream_t s, const uint16_t* x, const uint16_t* w, void* out, int N, int K, int max_tiles,
-                               const PipeGroups& groups, const char* what) {
+                               const PipeGroups& groups, const char* what, const RopeArgs& epilogue = RopeArgs{}) {
   constexpr int BM = 32 * WM * WAVES_M, BN = 32 * WN * WAVES_N;
   constexpr size_t lds = size_t(STAGES) * (BM + BN) * 128;
   static bool raised = false;
@@ -289,7 +289,7 @@ inline int launch_pipe_grouped(hipStream_t s, const uint16_t* x, const uint16_t*
   const long long blocks = (long long)max_tiles * (((MODE == kSilu ? 2 * N : N) + BN - 1) / BN);
   SP_REQUIRE(blocks < (1ll << 31), "%s: too many tiles", what);
   gemm_pipe_kernel<WM, WN, WAVES_M, WAVES_N, STAGES, MODE, bf16_t, uint16_t, true><<<dim3((unsigned)blocks), 64 * WAVES_M * WAVES_N, lds, s>>>(
-      x, w, nullptr, out, 0, N, K, K, RopeArgs{}, groups);
+      x, w, nullptr, out, 0, N, K, K, epilogue, groups);
   return check_launch(what);
 }
 

@@ -5,17 +5,20 @@
 namespace sprout {
 
 // out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T): a block's weight rows are half gate rows, half the matching up rows.
-int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K) {
+int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit) {
   const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
+  RopeArgs epi = {};
+  epi.act = act;
+  epi.limit = limit;
   int shape, splits;
   pipe_choice(T, 2 * I, K, false, &shape, &splits, true);
-  if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  if (shape == 1) return launch_pipe_mode<2, 2, 4, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  if (shape == 4) return launch_pipe_mode<1, 2, 2, 4, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  if (shape == 7) return launch_pipe_mode<1, 2, 2, 1, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
-  return launch_pipe_mode<1, 2, 4, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K);
+  if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);
+  if (shape == 1) return launch_pipe_mode<2, 2, 4, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);
+  if (shape == 4) return launch_pipe_mode<1, 2, 2, 4, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);
+  if (shape == 5) return launch_pipe_mode<1, 2, 2, 2, 3, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);
+  if (shape == 6) return launch_pipe_mode<6, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);
+  if (shape == 7) return launch_pipe_mode<1, 2, 2, 1, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);
+  return launch_pipe_mode<1, 2, 4, 2, 4, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);
 }
 
 // The block shape on which the rotating epilogue runs, or -1 where the plain product and a rotation kernel after

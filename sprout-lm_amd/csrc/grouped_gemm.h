@@ -22,6 +22,8 @@ struct GroupedArgs {
   int rows, tiles_per_group;
   int N, K;
   int up_offset;            // epilogue 1: weight row n is the gate's, row up_offset + n the matching up row
+  int act;                  // epilogue 1: which gated activation (GateAct), and its limit
+  float limit;
 };
 
 enum { kStore = 0, kGated = 1, kSigmoid = 2 };
@@ -34,8 +36,8 @@ int launch_grouped_mfma(hipStream_t s, int mode, int out_dtype, const GroupedArg
                         const char* what);
 
 // The pipelined tiled kernel in its grouped form (grouped_gemm_pipe.hip): tiles of 128 or 256 rows from a tile list,
-// K in whole steps of 64, bfloat16; `gated`: SiLU(gate) * up into bfloat16, else a float32 store.
-int grouped_pipe(hipStream_t s, bool gated, const void* x, const void* w, long long w_group_stride, const int32_t* tiles,
+// K in whole steps of 64, bfloat16; `gated`: act(gate, up) into bfloat16, else a float32 store.
+int grouped_pipe(hipStream_t s, bool gated, int act, float limit, const void* x, const void* w, long long w_group_stride, const int32_t* tiles,
                  const int32_t* n_tiles, int max_tiles, int tile_rows, const int32_t* gather, int gather_div, void* out,
                  int N, int K, const char* what);
 

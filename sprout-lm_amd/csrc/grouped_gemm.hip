@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void grouped_kernel(GroupedArgs p) {
       const int n = n0 + tx * 4 + j;
       if (n >= p.N) continue;
       float v = acc[i][j];
-      if (MODE == kGated) v = (v / (1.0f + expf(-v))) * acc2[i][j];
+      if (MODE == kGated) v = gated_value(v, acc2[i][j], p.act, p.limit);
       if (MODE == kSigmoid) v *= g;
       o[n] = from_float<TO>(v);
     }
@@ -128,7 +128,7 @@ static int grouped(hipStream_t s, int mode, int dtype, int out_dtype, const Grou
     if (p.tiles && tile_rows >= 128 && p.K % 64 == 0 && p.a_group_stride == 0 && p.a_stride == p.K &&
         ((mode == kGated && out_dtype == kBF16 && p.up_offset == p.N && p.out_stride == p.N) ||
          (mode == kStore && out_dtype == kF32 && p.out_stride == p.N)) && p.out_group_stride == 0)
-      return grouped_pipe(s, mode == kGated, p.a, p.w, p.w_group_stride, p.tiles, p.n_tiles, tiles, tile_rows, p.gather,
+      return grouped_pipe(s, mode == kGated, p.act, p.limit, p.a, p.w, p.w_group_stride, p.tiles, p.n_tiles, tiles, tile_rows, p.gather,
                           p.gather_div, p.out, p.N, p.K, what);
     return launch_grouped_mfma(s, mode, out_dtype, p, tiles, tile_rows, what);
   }
@@ -162,8 +162,8 @@ extern "C" int sp_head_gemm(void* stream, int dtype, const void* a, long long a_
 
 extern "C" int sp_expert_gate_up(void* stream, int dtype, const void* x, const void* w, const int32_t* tiles,
                                  const int32_t* n_tiles, int max_tiles, int tile_rows, const int32_t* pair_of_row, int top,
-                                 void* out, int T, int experts, int inner, int K, int activation) {
-  SP_REQUIRE(activation == 0, "sp_expert_gate_up: no kernel for activation %d (0 = SiLU)", activation);
+                                 void* out, int T, int experts, int inner, int K, int activation, float limit) {
+  SP_REQUIRE(activation >= 0 && activation < kGateActs, "sp_expert_gate_up: no kernel for activation %d", activation);
   SP_REQUIRE(T >= 0 && experts > 0 && inner > 0 && K > 0 && top > 0 && max_tiles > 0, "sp_expert_gate_up: bad sizes");
   SP_REQUIRE(x && w && tiles && n_tiles && pair_of_row && out, "sp_expert_gate_up: null operand");
   if (T == 0) return 0;
@@ -173,6 +173,7 @@ extern "C" int sp_expert_gate_up(void* stream, int dtype, const void* x, const v
   p.out = out; p.out_stride = inner;
   p.tiles = tiles; p.n_tiles = n_tiles;
   p.N = inner; p.K = K; p.up_offset = inner;
+  p.act = activation; p.limit = limit;
   return grouped((hipStream_t)stream, kGated, dtype, dtype, p, max_tiles, tile_rows, "sp_expert_gate_up");
 }
 

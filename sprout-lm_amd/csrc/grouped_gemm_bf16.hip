@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(GroupedArgs p) {
         const int n = n0 + wn + 32 * j + lr;
         if (n >= p.N) continue;
         float v = acc[i][j][r];
-        if (GATED) v = (v / (1.0f + expf(-v))) * acc2[i][j][r];
+        if (GATED) v = gated_value(v, acc2[i][j][r], p.act, p.limit);
         if (MODE == kSigmoid) v *= g;
         o[n] = from_float<TO>(v);
       }
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(256) void grouped_skinny_kernel(GroupedArgs p) {
     const int row = 4 * lj + r;
     if (row >= nrows) continue;
     float v = acc[r];
-    if (GATED) v = (v / (1.0f + expf(-v))) * acc2[r];
+    if (GATED) v = gated_value(v, acc2[r], p.act, p.limit);
     if (MODE == kSigmoid)
       v *= 1.0f / (1.0f + expf(-to_float(((const bf16_t*)p.gate)[(long long)(row0 + row) * p.gate_stride + group])));
     ((TO*)p.out)[(long long)(row0 + row) * p.out_stride + group * p.out_group_stride + n] = from_float<TO>(v);

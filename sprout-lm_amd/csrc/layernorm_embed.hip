@@ -1,17 +1,17 @@
-// Layer norm without bias, and the token embedding with a hashed-pair (bigram) table added.
+// Layer norm (bias optional), and the token embedding with a hashed-pair (bigram) table added.
 // All arithmetic is float32; only loads and stores see the storage type.
 #include "common.h"
 #include "sprout_hip.h"
 
 namespace sprout {
 
-// y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w.  One block a row; the row is read three times (the second
+// y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w (+ b where b is given).  One block a row; the row is read three times (the second
 // and third time from the caches): the variance is the mean of the squared deviations, not E[x^2] - mean^2.
 // With w2 and out2 the same normalised row is also written times a second weight (two norms of one input).
 template <typename TW, typename TO>
 __global__ void layernorm_kernel(const float* __restrict__ x, const int32_t* __restrict__ rows,
-                                 const TW* __restrict__ w, const TW* __restrict__ w2, float eps, TO* __restrict__ out,
-                                 TO* __restrict__ out2, int H) {
+                                 const TW* __restrict__ w, const TW* __restrict__ w2, const TW* __restrict__ b,
+                                 const TW* __restrict__ b2, float eps, TO* __restrict__ out, TO* __restrict__ out2, int H) {
   __shared__ float scratch[16];
   const int r = blockIdx.x;
   const float* in = x + size_t(rows ? rows[r] : r) * H;
@@ -40,8 +40,8 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int32_t* __r
       const int i = threadIdx.x + j * blockDim.x;
       if (i >= H) continue;
       const float y = (v[j] - mean) * scale;
-      o[i] = from_float<TO>(y * to_float(w[i]));
-      if (o2) o2[i] = from_float<TO>(y * to_float(w2[i]));
+      o[i] = from_float<TO>(fmaf(y, to_float(w[i]), b ? to_float(b[i]) : 0.f));
+      if (o2) o2[i] = from_float<TO>(fmaf(y, to_float(w2[i]), b2 ? to_float(b2[i]) : 0.f));
     }
     return;
   }
@@ -56,8 +56,8 @@ __global__ void layernorm_kernel(const float* __restrict__ x, const int32_t* __r
   const float scale = 1.0f / sqrtf(block_sum(sq, scratch) / float(H) + eps);
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     const float y = (in[i] - mean) * scale;
-    o[i] = from_float<TO>(y * to_float(w[i]));
-    if (o2) o2[i] = from_float<TO>(y * to_float(w2[i]));
+    o[i] = from_float<TO>(fmaf(y, to_float(w[i]), b ? to_float(b[i]) : 0.f));
+    if (o2) o2[i] = from_float<TO>(fmaf(y, to_float(w2[i]), b2 ? to_float(b2[i]) : 0.f));
   }
 }
 
@@ -103,14 +103,16 @@ __global__ void embed_bigram_kernel(const TW* __restrict__ table, const TW* __re
 using namespace sprout;
 
 extern "C" int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, const void* w2,
-                            float eps, int out_dtype, void* out, void* out2, int R, int H) {
+                            const void* b, const void* b2, float eps, int out_dtype, void* out, void* out2, int R, int H) {
   SP_REQUIRE(R >= 0 && H > 0 && x && w && out, "sp_layernorm: bad arguments R=%d H=%d", R, H);
   SP_REQUIRE((w2 == nullptr) == (out2 == nullptr), "sp_layernorm: a second weight goes with a second output");
+  SP_REQUIRE(!b2 || w2, "sp_layernorm: a second bias goes with a second weight");
   if (R == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
   const int threads = H >= 2048 ? 512 : 256;
 #define SP_LN(TW, TO) \
-  layernorm_kernel<TW, TO><<<R, threads, 0, s>>>(x, rows, (const TW*)w, (const TW*)w2, eps, (TO*)out, (TO*)out2, H)
+  layernorm_kernel<TW, TO><<<R, threads, 0, s>>>(x, rows, (const TW*)w, (const TW*)w2, (const TW*)b, (const TW*)b2, eps, \
+                                                (TO*)out, (TO*)out2, H)
   if (w_dtype == kF32 && out_dtype == kF32) SP_LN(float, float);
   else if (w_dtype == kF32 && out_dtype == kBF16) SP_LN(float, bf16_t);
   else if (w_dtype == kBF16 && out_dtype == kF32) SP_LN(bf16_t, float);

@@ -4,7 +4,8 @@
 // Variants of an operation that parts may ask for are numbered, one `int` each; a number that no kernel
 // implements is refused with an error, so another variant is an addition here and in the kernels, never a guess:
 //   pairing of a rotation     0 = halves of the rotated dimensions (d with d + rotary_dim / 2, "neox")
-//   activation of a gated product   0 = SiLU (x / (1 + exp(-x)))
+//   activation of a gated product   0 = SiLU(g) * u (x / (1 + exp(-x)));  1 = clamped: g' = min(g, limit),
+//                                   u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1)
 #pragma once
 #include <stdint.h>
 
@@ -55,7 +56,7 @@ int sp_qkv_rope_cache(void* stream, const void* x, const float* residual, int no
 int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T);
 // out [T, I] = silu(x . w[:I]^T) * (x . w[I:]^T)
 int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
-                    const void* w, void* out, int T, int I, int K, int activation);
+                    const void* w, void* out, int T, int I, int K, int activation, float limit);
 
 // Rotates q and k heads of qkv[T, (nq + 2 nkv) * hd] in place (neox pairing, angle = position *
 // inv_freq[d]) and writes k and v of every token into the paged pools at slot_mapping[t]
@@ -83,13 +84,17 @@ int sp_attention_plan(int dtype, int hd, int page_size, int nq, int nkv, int ker
 int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
                                       int n_decode, int max_decode_ctx, int n_tiles, int max_tile_ctx);
 // scores: what stands between q . k and the softmax, numbered like the variants above: 0 = the scaled product and
-// nothing else (the one the kernels have; a cap, a bias or sinks would be further numbers, refused until written).
+// nothing else; 1 = the scaled product s squashed to softcap * tanh(s / softcap).  sinks (null: none): one float per
+// query head whose exponential joins the softmax's denominator: a term without key or value, neither scaled nor
+// capped.  mask_chunk > 0: a query sees only the keys of its own block of mask_chunk positions, counted from
+// position 0 of the sequence (beside the window, if both are given).
 int sp_attention(void* stream, int dtype, const void* q, int q_stride, const void* k_pool,
                  const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                  const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, int tile_q,
                  int max_tile_ctx, int mean_tile_walk, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                  float* workspace, int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size,
-                 int num_pages, int window, float scale, int kernel_kind, int scores);
+                 int num_pages, int window, float scale, int kernel_kind, int scores, float softcap, const float* sinks,
+                 int mask_chunk);
 
 // A step of one-query sequences only (bfloat16): attention with the output projection folded into the merge
 // of the key chunks: residual[q_start[seq], :] += attention(seq) . w_o^T with w_o [hidden, nq * hd] bfloat16
@@ -102,10 +107,23 @@ int sp_attention_decode_project(void* stream, const void* q, int q_stride, const
                                 const int32_t* ctx_len, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                                 float* workspace, int64_t workspace_floats, const void* w_o, float* residual,
                                 int hidden, int nq, int nkv, int hd, int page_size, int num_pages, int window,
-                                float scale, int scores);
+                                float scale, int scores, float softcap, const float* sinks, int mask_chunk);
 
-// out[t, i] = act(gu[t, i]) * gu[t, I + i]
-int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation);
+// out[t, i] = act(gu[t, i], gu[t, I + i]) (times sigmoid(row_gate[t * row_gate_stride]) where row_gate, float32, is given)
+int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I, int activation, float limit,
+                const float* row_gate, long long row_gate_stride);
+
+// Between the q/k/v projection and attention where keys and values differ in width (both are kept `width` wide, zeros
+// behind) or q and k are normed as whole rows.  proj [T, stride] holds q (nq * dim), k (nkv * dim), v (nkv * vdim).
+// q_norm / k_norm (both or neither): RMS norm over the whole q row and the whole k row times these weights, eps inside
+// the root.  The first rotary_dim numbers of every q and k head turn (d with d + rotary_dim / 2) by positions *
+// inv_freq (+ inv_freq_tail: in float64).  blend (one number lambda of `dtype`): v <- (1 - lambda) v + lambda first[t];
+// keep_first: first[t] <- v instead.  q to q_out [T, nq * width]; k and v into the pools at slot_mapping (null or
+// negative: not cached), keys [pages][nkv][page][width], values [pages][nkv][width][page].
+int sp_qkv_prepare(void* stream, int dtype, const void* proj, long long stride, int nq, int nkv, int dim, int vdim, int width,
+                   const void* q_norm, const void* k_norm, float eps, const int32_t* positions, const float* inv_freq,
+                   const float* inv_freq_tail, int rotary_dim, const void* blend, void* first, int keep_first,
+                   const int32_t* slot_mapping, void* k_pool, void* v_pool, int page_size, int num_pages, void* q_out, int T);
 
 // dst (dst_dtype) = src (src_dtype), n elements
 
@@ -118,7 +136,7 @@ int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I
 //                          q_out [T, nq * hd], k and v into the paged pools at slot_mapping.  Head sizes in 16s.
 int sp_gate_up_silu_f32_takes(int T, int I, int K);
 int sp_gate_up_silu_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, float* out,
-                        int T, int I, int K, int activation);
+                        int T, int I, int K, int activation, float limit);
 int sp_qkv_rope_cache_f32_takes(int T, int K, int nq, int nkv, int hd, int rotary_dim, int pairing);
 int sp_qkv_rope_cache_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, int bias_dtype,
                           const void* bias, float* q_out, const int32_t* positions, const float* inv_freq,
@@ -155,10 +173,11 @@ int sp_sample_static(void* stream, const float* logits, const float* temperature
                      const int32_t* counter, int32_t* out, int R, int V);
 int sp_sample_static_max_floats();
 
-// Layer norm without bias: out[r, :] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w, x float32 [*, H], rows as in
-// sp_rmsnorm.  With w2 and out2 (both or neither) the normalised row is also written times a second weight.
-int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, const void* w2, float eps,
-                 int out_dtype, void* out, void* out2, int R, int H);
+// Layer norm: out[r, :] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w (+ b where b is given, of w's dtype),
+// x float32 [*, H], rows as in sp_rmsnorm.  With w2 and out2 (both or neither; b2 optional) the normalised row is also
+// written times a second weight.
+int sp_layernorm(void* stream, const float* x, const int32_t* rows, int w_dtype, const void* w, const void* w2,
+                 const void* b, const void* b2, float eps, int out_dtype, void* out, void* out2, int R, int H);
 
 // residual[t, :] = table[tokens[t], :] + pairs[row, :] with row = (previous * mul_prev + tokens[t] * mul_cur) mod buckets,
 // and row `buckets` (the table's last) at position 0.  The token before a step's first token of a sequence is read
@@ -206,7 +225,7 @@ int sp_route_sort(void* stream, const int32_t* ids, int pairs, int experts, int 
                   int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
 int sp_expert_gate_up(void* stream, int dtype, const void* x, const void* w, const int32_t* tiles, const int32_t* n_tiles,
                       int max_tiles, int tile_rows, const int32_t* pair_of_row, int top, void* out, int T, int experts,
-                      int inner, int K, int activation);
+                      int inner, int K, int activation, float limit);
 int sp_expert_down(void* stream, int dtype, const void* act, const void* w, const int32_t* tiles, const int32_t* n_tiles,
                    int max_tiles, int tile_rows, float* out, int rows, int experts, int hidden, int inner);
 // sp_route: sp_route_topk and sp_route_sort in one call (one launch up to 256 tokens).
@@ -214,6 +233,17 @@ int sp_route(void* stream, const float* logits, int32_t* ids, float* weights, in
              int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
 int sp_route_combine(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,
                      float* residual, int T, int H);
+// sp_route with another rule of choice: scores = the softmax over all `outputs` logits of a token (rows `stride`
+// apart); the choice goes by score + correction[e] (null: none) and only among the outputs of the `keep` of `groups`
+// equal groups of neighbours whose best such sum is largest (the lower index wins every tie); weights = the chosen
+// outputs' scores times `scale`.  Outputs from `real` on have no weights of their own (they return the token's input):
+// they get rows but no tiles.  Up to 256 outputs.  sp_route_combine_identity is the weighted sum that goes with it: a
+// choice whose id is `real` or more adds weight * x[t] (x [T, H] of x_dtype) instead of an output row.
+int sp_route_scored(void* stream, const float* logits, long long stride, const float* correction, int groups, int keep,
+                    float scale, int32_t* ids, float* weights, int T, int outputs, int real, int top, int tile_rows,
+                    int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
+int sp_route_combine_identity(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,
+                              const int32_t* ids, int x_dtype, const void* x, int real, float* residual, int T, int H);
 
 // Probes for the benchmark's report, not used by the engine: a kernel that only reads `bytes` of `data` (16-byte
 // loads from `blocks` blocks of 256 threads), and one that only multiplies on the matrix cores (`blocks` blocks of four waves,

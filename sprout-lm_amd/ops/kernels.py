@@ -63,8 +63,10 @@ def _ptr(t):
 # kernels; anything else is refused (KernelError) before a launch.
 ROTARY_PAIRINGS = {"halves": 0}          # dimension d turns with d + rotary_dim / 2 ("neox"); the latent mixer's own
                                          # kernel (latent_prepare) turns neighbours (2i, 2i + 1)
-GATE_ACTIVATIONS = {"silu": 0}
-SCORE_STAGES = {"scaled_dot": 0}         # what stands between q . k and the softmax: the scale and nothing else
+GATE_ACTIVATIONS = {"silu": 0,           # silu(g) * u
+                    "clamped_swish": 1}  # g' = min(g, limit), u' = clamp(u, -limit, limit): g' * sigmoid(1.702 g') * (u' + 1)
+SCORE_STAGES = {"scaled_dot": 0,         # what stands between q . k and the softmax: the scale and nothing else,
+                "capped": 1}             # or the scaled product s squashed to cap * tanh(s / cap)
 MAX_HEAD_DIM = 512                       # the largest head size any attention kernel takes
 
 
@@ -123,9 +125,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
 
 
 def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, rows: torch.Tensor | None = None,
-              weight2: torch.Tensor | None = None, out2: torch.Tensor | None = None) -> None:
-    """out[r] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight of x[rows[r]] or x[r]; x is float32.  With weight2
-    and out2 the same normalised row times a second weight goes to out2 (two norms of one input in one pass)."""
+              weight2: torch.Tensor | None = None, out2: torch.Tensor | None = None, bias: torch.Tensor | None = None,
+              bias2: torch.Tensor | None = None) -> None:
+    """out[r] = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight (+ bias) of x[rows[r]] or x[r]; x is float32.  With
+    weight2 and out2 the same normalised row times a second weight (+ bias2) goes to out2 (two norms of one input in one
+    pass)."""
     _gpu(x, "norm input"); _gpu(weight, "norm weight"); _gpu(out, "norm output")
     R, H = out.shape
     if x.dtype != torch.float32 or x.shape[1] != H or weight.numel() != H:
@@ -136,12 +140,20 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tens
         _gpu(weight2, "second norm weight"); _gpu(out2, "second norm output")
         if weight2.dtype != weight.dtype or weight2.numel() != H or out2.dtype != out.dtype or tuple(out2.shape) != (R, H):
             raise KernelError("layernorm: the second weight and output must be shaped and typed like the first")
+    for b, what in ((bias, "norm bias"), (bias2, "second norm bias")):
+        if b is not None:
+            _gpu(b, what)
+            if b.dtype != weight.dtype or b.numel() != H:
+                raise KernelError(f"layernorm: the {what} must be shaped and typed like the weight")
+    if bias2 is not None and weight2 is None:
+        raise KernelError("layernorm: a second bias goes with a second weight")
     if rows is not None:
         _ints(rows, R, "norm rows")
     elif x.shape[0] < R:
         raise KernelError("layernorm: fewer input rows than output rows")
     check(library().sp_layernorm(_stream(), x.data_ptr(), _ptr(rows), _code(weight, "norm weight"), weight.data_ptr(),
-                                 _ptr(weight2), float(eps), _code(out, "norm output"), out.data_ptr(), _ptr(out2), R, H))
+                                 _ptr(weight2), _ptr(bias), _ptr(bias2), float(eps), _code(out, "norm output"),
+                                 out.data_ptr(), _ptr(out2), R, H))
 
 
 def embed_bigram(table: torch.Tensor, pairs: torch.Tensor, tokens, positions, q_start, q_len, seq_of_token, state_slots,
@@ -264,7 +276,7 @@ def route_sort(ids: torch.Tensor, experts: int, row_of_pair, pair_of_row, tiles,
 
 
 def expert_gate_up(x: torch.Tensor, w: torch.Tensor, tiles, n_tiles, pair_of_row, top: int, out: torch.Tensor,
-                   activation: str = "silu", tile_rows: int = 64) -> None:
+                   activation: str = "silu", tile_rows: int = 64, limit: float = 0.0) -> None:
     """out[row] = act(x[token] . w[e, :I]^T) * (x[token] . w[e, I:]^T) for every sorted row (w [experts, 2 I, K])."""
     _gpu(x, "expert input"); _gpu(w, "expert gate/up weights"); _gpu(out, "expert activations")
     T, K = x.shape
@@ -275,7 +287,8 @@ def expert_gate_up(x: torch.Tensor, w: torch.Tensor, tiles, n_tiles, pair_of_row
     _ints(tiles, 3 * max_tiles, "expert tiles"); _ints(n_tiles, 1, "tile count"); _ints(pair_of_row, T * top, "pair_of_row")
     check(library().sp_expert_gate_up(_stream(), _code(w, "expert weights"), x.data_ptr(), w.data_ptr(), tiles.data_ptr(),
                                       n_tiles.data_ptr(), max_tiles, tile_rows, pair_of_row.data_ptr(), top, out.data_ptr(),
-                                      T, E, two_i // 2, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+                                      T, E, two_i // 2, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation"),
+                                      float(limit)))
 
 
 def expert_down(act: torch.Tensor, w: torch.Tensor, tiles, n_tiles, out: torch.Tensor, tile_rows: int = 64) -> None:
@@ -302,6 +315,85 @@ def route_combine(y: torch.Tensor, row_of_pair, weights: torch.Tensor, residual:
     _ints(row_of_pair, T * top, "row_of_pair")
     check(library().sp_route_combine(_stream(), y.data_ptr(), row_of_pair.data_ptr(), weights.data_ptr(), top,
                                      residual.data_ptr(), T, H))
+
+
+def route_scored(logits: torch.Tensor, outputs: int, real: int, correction, groups: int, keep: int, scale: float,
+                 ids: torch.Tensor, weights: torch.Tensor, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows: int = 64) -> None:
+    """Choice and order by another rule: scores = the softmax over the first `outputs` columns of a row of logits; the
+    choice goes by score + correction and only inside the `keep` best of `groups` groups of neighbours; weights = the
+    chosen scores times `scale`.  Outputs from `real` on are identity outputs: rows, but no tiles (see sprout_hip.h)."""
+    _gpu(logits, "router logits"); _gpu(ids, "chosen experts"); _gpu(weights, "expert weights")
+    T, stride = logits.shape
+    top = ids.shape[1]
+    if logits.dtype != torch.float32 or ids.dtype != torch.int32 or weights.dtype != torch.float32 or \
+            tuple(ids.shape) != (T, top) or tuple(weights.shape) != (T, top) or not 0 < top <= outputs <= stride:
+        raise KernelError("route_scored: float32 logits [T, >= outputs], int32 ids and float32 weights [T, top] expected")
+    if correction is not None:
+        _gpu(correction, "router correction")
+        if correction.dtype != torch.float32 or correction.numel() != outputs:
+            raise KernelError(f"route_scored: the correction must hold {outputs} float32 values")
+    pairs = T * top
+    _ints(row_of_pair, pairs, "row_of_pair"); _ints(pair_of_row, pairs, "pair_of_row")
+    _ints(tiles, 3 * route_max_tiles(pairs, real, tile_rows), "expert tiles"); _ints(n_tiles, 1, "tile count")
+    check(library().sp_route_scored(_stream(), logits.data_ptr(), stride, _ptr(correction), int(groups), int(keep), float(scale),
+                                    ids.data_ptr(), weights.data_ptr(), T, outputs, real, top, tile_rows,
+                                    row_of_pair.data_ptr(), pair_of_row.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr()))
+
+
+def route_combine_identity(y: torch.Tensor, row_of_pair, ids: torch.Tensor, weights: torch.Tensor, x: torch.Tensor, real: int,
+                           residual: torch.Tensor) -> None:
+    """residual[t] += sum_k weights[t, k] * (y[row_of_pair[t * top + k]] if ids[t, k] < real else x[t])."""
+    _gpu(y, "expert outputs"); _gpu(weights, "expert weights"); _gpu(residual, "residual"); _gpu(x, "expert input")
+    T, top = weights.shape
+    H = residual.shape[1]
+    if y.dtype != torch.float32 or tuple(y.shape) != (T * top, H) or residual.dtype != torch.float32 or residual.shape[0] < T \
+            or weights.dtype != torch.float32 or x.shape[0] < T or x.shape[1] != H:
+        raise KernelError("route_combine_identity: float32 outputs [T * top, H], weights [T, top], inputs and residual [T, H] expected")
+    _ints(row_of_pair, T * top, "row_of_pair"); _ints(ids, T * top, "chosen experts")
+    check(library().sp_route_combine_identity(_stream(), y.data_ptr(), row_of_pair.data_ptr(), weights.data_ptr(), top,
+                                              ids.data_ptr(), _code(x, "expert input"), x.data_ptr(), int(real),
+                                              residual.data_ptr(), T, H))
+
+
+def qkv_prepare(proj: torch.Tensor, nq: int, nkv: int, dim: int, vdim: int, width: int, q_out: torch.Tensor, positions=None,
+                inv_freq=None, inv_freq_tail=None, rotary_dim: int = 0, q_norm=None, k_norm=None, eps: float = 0.0,
+                blend=None, first=None, keep_first: bool = False, slot_mapping=None, k_pool=None, v_pool=None) -> None:
+    """From rows of projections [q | k | v] (heads of `dim`, `dim` and `vdim` numbers): optional RMS norm over the whole
+    q row and the whole k row, optional rotation of the heads' first rotary_dim numbers, optional blend of the values
+    with `first` (or `first` <- values), q to q_out [T, nq * width], k and v into pools that keep both `width` wide
+    (zeros behind); see sprout_hip.h."""
+    _gpu(proj, "projections"); _gpu(q_out, "queries")
+    T, stride = proj.shape
+    if stride < (nq + nkv) * dim + nkv * vdim or tuple(q_out.shape) != (T, nq * width) or q_out.dtype != proj.dtype:
+        raise KernelError(f"qkv_prepare: rows of {stride} and queries {tuple(q_out.shape)} {q_out.dtype} do not fit the head sizes")
+    if (q_norm is None) != (k_norm is None):
+        raise KernelError("qkv_prepare: queries and keys are normed together or not at all")
+    if q_norm is not None:
+        _gpu(q_norm, "query norm"); _gpu(k_norm, "key norm")
+        if q_norm.dtype != proj.dtype or k_norm.dtype != proj.dtype or q_norm.numel() != nq * dim or k_norm.numel() != nkv * dim:
+            raise KernelError("qkv_prepare: the norm weights must cover the whole q row and the whole k row")
+    if rotary_dim:
+        _ints(positions, T, "positions"); _gpu(inv_freq, "inv_freq")
+        if inv_freq.dtype != torch.float32 or inv_freq.numel() < rotary_dim // 2 or rotary_dim % 2 or rotary_dim > dim:
+            raise KernelError("qkv_prepare: inv_freq must hold rotary_dim / 2 float32 values, rotary_dim even and at most dim")
+        if inv_freq_tail is not None and (inv_freq_tail.dtype != torch.float32 or inv_freq_tail.numel() != inv_freq.numel()):
+            raise KernelError("qkv_prepare: inv_freq_tail must be float32 and as long as inv_freq")
+    if blend is not None or keep_first:
+        _gpu(first, "first values")
+        if first.dtype != proj.dtype or first.shape[0] < T or first.shape[1] != nkv * vdim:
+            raise KernelError(f"qkv_prepare: the first layer's values must be [>= {T}, {nkv * vdim}] {proj.dtype}")
+        if blend is not None and (blend.dtype != proj.dtype or blend.numel() != 1 or not blend.is_cuda):
+            raise KernelError("qkv_prepare: the blend factor is one number of the projections' dtype on the GPU")
+    page_size = num_pages = 0
+    if slot_mapping is not None:
+        _ints(slot_mapping, T, "slot_mapping")
+        num_pages, page_size = _check_pools(k_pool, v_pool, nkv, width, proj.dtype, "qkv_prepare")
+    check(library().sp_qkv_prepare(_stream(), _code(proj, "projections"), proj.data_ptr(), stride, nq, nkv, dim, vdim, width,
+                                   _ptr(q_norm), _ptr(k_norm), float(eps), _ptr(positions) if rotary_dim else None,
+                                   _ptr(inv_freq) if rotary_dim else None, _ptr(inv_freq_tail) if rotary_dim else None,
+                                   int(rotary_dim), _ptr(blend), _ptr(first), int(bool(keep_first)), _ptr(slot_mapping),
+                                   _ptr(k_pool) if slot_mapping is not None else None,
+                                   _ptr(v_pool) if slot_mapping is not None else None, page_size, num_pages, q_out.data_ptr(), T))
 
 
 STORE, ACCUMULATE, STORE_F32 = 0, 1, 2
@@ -426,16 +518,27 @@ def attention_plan(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: in
 
 def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor,
               batch: AttentionBatch, out: torch.Tensor, nq: int, nkv: int, hd: int, window: int | None, scale: float,
-              workspace=None, kind: int = 0, project=None, scores: str = "scaled_dot") -> bool:
+              workspace=None, kind: int = 0, project=None, scores: str = "scaled_dot", softcap: float = 0.0,
+              sinks: torch.Tensor | None = None, mask_chunk: int | None = None) -> bool:
     """Causal attention of a mixed batch over paged keys and values (see sprout_hip.h).
 
     `workspace(n)` must return a float32 device tensor of at least n elements (default: a new one).
+    `scores`: "scaled_dot", or "capped" (the scaled product s becomes softcap * tanh(s / softcap)).  `sinks`: float32
+    [nq], one logit per query head that joins the softmax's denominator without a key or value.  `mask_chunk`: a
+    query sees only the keys of its own block of that many positions, counted from position 0.
     `project`: (w_o [hidden, nq * hd], residual float32 [T, hidden]) of an output projection without bias
     that may be folded in: where the kernels take the step that way (one-query sequences only, bfloat16),
     residual += attention . w_o^T, `out` is left untouched and True is returned; otherwise False, and the
     projection is the caller's.
     """
     scores_code = variant_code(SCORE_STAGES, scores, "score stage")
+    if scores_code == 1 and not softcap > 0.0:
+        raise KernelError("attention: capped scores need a positive cap")
+    if sinks is not None:
+        _gpu(sinks, "sinks")
+        if sinks.dtype != torch.float32 or sinks.numel() != nq:
+            raise KernelError(f"attention: sinks must be {nq} float32 values")
+    stage = (float(softcap), _ptr(sinks), int(mask_chunk) if mask_chunk else 0)
     for t, what in ((q, "q"), (out, "attention output")):
         _gpu(t, what)
     T = out.shape[0]
@@ -494,7 +597,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                 block_tables.shape[1], batch.q_start.data_ptr(), batch.ctx_len.data_ptr(),
                 _ptr(decode) if decode is not None else None, n_decode, max_decode_ctx, _ptr(ws), need, w_o.data_ptr(),
                 residual.data_ptr(), hidden, nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
-                float(scale), scores_code))
+                float(scale), scores_code, *stage))
             return True
     check(library().sp_attention(_stream(), _code(q, "q"), q.data_ptr(), q_stride, k_pool.data_ptr(), v_pool.data_ptr(),
                                  block_tables.data_ptr(), block_tables.shape[1], batch.q_start.data_ptr(),
@@ -503,7 +606,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                                  _ptr(decode) if n_decode and decode is not None else None, n_decode,
                                  max_decode_ctx, _ptr(ws),
                                  need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
-                                 float(scale), kind, scores_code))
+                                 float(scale), kind, scores_code, *stage))
     return False
 
 
@@ -613,7 +716,7 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tenso
 
 
 def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0,
-                 activation: str = "silu") -> None:
+                 activation: str = "silu", limit: float = 0.0) -> None:
     """out = act(a . w[:I]^T) * (a . w[I:]^T) for activations a as in `qkv_rope_cache`."""
     _gpu(w, "gate/up weight"); _gpu(out, "gated output")
     N, K = w.shape
@@ -621,11 +724,11 @@ def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm
     if w.dtype != torch.bfloat16 or N % 2 or tuple(out.shape) != (T, N // 2) or out.dtype != torch.bfloat16:
         raise KernelError("gate_up_silu: weight [2 I, K] and output [T, I] bfloat16 expected")
     check(library().sp_gate_up_silu(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(), out.data_ptr(), T, N // 2, K,
-                                    variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+                                    variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit)))
 
 
 def gate_up_silu_f32(w: torch.Tensor, x: torch.Tensor, out: torch.Tensor, activation: str = "silu", norm_weight=None,
-                     eps: float = 0.0) -> bool:
+                     eps: float = 0.0, limit: float = 0.0) -> bool:
     """out = act(a . w[:I]^T) * (a . w[I:]^T), everything float32, for the few tokens of a decode step; a = x, or
     rmsnorm(x) * norm_weight computed inside the kernel where norm_weight is given (x is then the residual).  Returns
     False (and does nothing) where the kernel does not take the shape: the caller then multiplies and gates in turn."""
@@ -638,7 +741,7 @@ def gate_up_silu_f32(w: torch.Tensor, x: torch.Tensor, out: torch.Tensor, activa
         return False
     _gpu(w, "gate/up weight"); _gpu(x, "activations"); _gpu(out, "gated output")
     check(library().sp_gate_up_silu_f32(_stream(), x.data_ptr(), _ptr(norm_weight), float(eps), w.data_ptr(), out.data_ptr(),
-                                        T, I, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+                                        T, I, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit)))
     return True
 
 
@@ -676,14 +779,22 @@ def qkv_rope_cache_f32(w: torch.Tensor, bias, x: torch.Tensor, q_out: torch.Tens
     return True
 
 
-def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
-    """out[t, i] = act(gu[t, i]) * gu[t, I + i]."""
+def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu", limit: float = 0.0,
+             row_gate: torch.Tensor | None = None, row_gate_column: int = 0) -> None:
+    """out[t, i] = act(gu[t, i], gu[t, I + i]), times sigmoid(row_gate[t, row_gate_column]) where row_gate (float32
+    [T, *]) is given."""
     _gpu(gu, "gate/up"); _gpu(out, "gated output")
     T, I = out.shape
     if tuple(gu.shape) != (T, 2 * I) or gu.dtype != out.dtype:
         raise KernelError(f"silu_mul: shapes do not fit: gu {tuple(gu.shape)}, out {tuple(out.shape)}")
+    gate_ptr, gate_stride = None, 0
+    if row_gate is not None:
+        _gpu(row_gate, "row gate")
+        if row_gate.dtype != torch.float32 or row_gate.dim() != 2 or row_gate.shape[0] < T or not 0 <= row_gate_column < row_gate.shape[1]:
+            raise KernelError("silu_mul: the row gate must be float32 [>= T, columns]")
+        gate_ptr, gate_stride = row_gate.data_ptr() + 4 * row_gate_column, row_gate.shape[1]
     check(library().sp_silu_mul(_stream(), _code(gu, "gate/up"), gu.data_ptr(), out.data_ptr(), T, I,
-                                variant_code(GATE_ACTIVATIONS, activation, "gate activation")))
+                                variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit), gate_ptr, gate_stride))
 
 
 def random_fill(dst: torch.Tensor, key: int, scale: float, offset: float | None = None, first: int = 0) -> None:

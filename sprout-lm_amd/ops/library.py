@@ -24,11 +24,11 @@ def _declare(lib):
                           c_int, c_int, c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
                          c_int, c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_float, c_int, c_int],
+                         c_int, c_int, c_float, c_int, c_int, c_float, c_void, c_int],
         "sp_attention_decode_project_takes": [c_int] * 7,
         "sp_attention_decode_project": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void,
                                         c_int, c_int, c_void, c_i64, c_void, c_void, c_int, c_int, c_int, c_int, c_int,
-                                        c_int, c_int, c_float, c_int],
+                                        c_int, c_int, c_float, c_int, c_float, c_void, c_int],
         "sp_attention_plan": [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(c_int)],
         "sp_fused_supported": [c_int] * 8,
         "sp_fused_norm_pays": [c_int] * 3,
@@ -39,18 +39,18 @@ def _declare(lib):
         "sp_qkv_rope_cache": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_void, c_void,
                               c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_int],
         "sp_rope_table": [c_void, c_void, c_void, c_int, c_void, c_int],
-        "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int],
+        "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int, c_float],
         "sp_gate_up_silu_f32_takes": [c_int, c_int, c_int],
-        "sp_gate_up_silu_f32": [c_void, c_void, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int],
+        "sp_gate_up_silu_f32": [c_void, c_void, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int, c_float],
         "sp_qkv_rope_cache_f32_takes": [c_int] * 7,
         "sp_qkv_rope_cache_f32": [c_void, c_void, c_void, c_float, c_void, c_int, c_void, c_void, c_void, c_void, c_void,
                                   c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int],
-        "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int, c_int],
+        "sp_silu_mul": [c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_float, c_void, c_i64],
         "sp_sample": [c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_sample_workspace_floats": [c_int, c_int],
         "sp_feed_tokens": [c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_random_fill": [c_void, c_int, c_void, c_i64, ctypes.c_uint64, c_i64, c_float, c_float, c_int],
-        "sp_layernorm": [c_void, c_void, c_void, c_int, c_void, c_void, c_float, c_int, c_void, c_void, c_int, c_int],
+        "sp_layernorm": [c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void, c_float, c_int, c_void, c_void, c_int, c_int],
         "sp_embed_bigram": [c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_void,
                             c_int, c_int, c_int, c_i64, c_i64, c_i64],
         "sp_latent_prepare": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_float,
@@ -63,7 +63,12 @@ def _declare(lib):
         "sp_route": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_void, c_void, c_void],
         "sp_route_sort": [c_void, c_void, c_int, c_int, c_int, c_void, c_void, c_void, c_void],
         "sp_expert_gate_up": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_void, c_int, c_void, c_int,
-                              c_int, c_int, c_int, c_int],
+                              c_int, c_int, c_int, c_int, c_float],
+        "sp_route_scored": [c_void, c_void, c_i64, c_void, c_int, c_int, c_float, c_void, c_void, c_int, c_int, c_int, c_int,
+                            c_int, c_void, c_void, c_void, c_void],
+        "sp_route_combine_identity": [c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_void, c_int, c_void, c_int, c_int],
+        "sp_qkv_prepare": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_int, c_void, c_void, c_float, c_void,
+                           c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_void, c_int],
         "sp_expert_down": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_int],
         "sp_route_combine": [c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int],
         "sp_probe_read": [c_void, c_void, c_i64, c_int, c_void],

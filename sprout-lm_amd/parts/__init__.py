@@ -1,6 +1,6 @@
 from .base import (Block, FeedForward, Mixer, Norm, NormFold, Part, PositionEncoding, make_part, register_part,
                    registered_parts)
-from . import attention, block, embedding, latent_attention, mlp, moe, norm, rotary  # noqa: F401  (register the built-in parts)
+from . import attention, block, embedding, latent_attention, mlp, moe, norm, rotary, sink_attention  # noqa: F401  (register the built-in parts)
 
 __all__ = ["Block", "FeedForward", "Mixer", "Norm", "NormFold", "Part", "PositionEncoding", "make_part", "register_part",
            "registered_parts"]

@@ -6,17 +6,21 @@ from .base import Block, register_part
 
 @register_part("block", "pre_norm")
 class PreNormBlock(Block):
-    """x += mixer(norm(x)); x += feed_forward(norm(x)).  The residual stream x is float32."""
+    """x += mixer(norm(x)); x += feed_forward(norm(x)).  The residual stream x is float32.  `ffn` (and its norm) may
+    be absent: the layer is then its mixer alone."""
 
     graph_safe = True
 
     graph_safe_portions = True
 
-    def __init__(self, mixer_norm, mixer, ffn_norm, ffn):
+    def __init__(self, mixer_norm, mixer, ffn_norm=None, ffn=None):
         self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
 
     def parts(self):
-        return {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "ffn_norm": self.ffn_norm, "ffn": self.ffn}
+        named = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.ffn is not None:
+            named.update({"ffn_norm": self.ffn_norm, "ffn": self.ffn})
+        return named
 
     def forward(self, ctx, residual, caches):
         T, H = residual.shape
@@ -25,6 +29,8 @@ class PreNormBlock(Block):
         if not self.mixer.forward_from_residual(ctx, self.mixer_norm, residual, cache):
             self.mixer_norm.forward(ctx, residual, h)
             self.mixer.forward(ctx, h, residual, cache)
+        if self.ffn is None:
+            return
         if not self.ffn.forward_from_residual(ctx, self.ffn_norm, residual):
             self.ffn_norm.forward(ctx, residual, h)
             self.ffn.forward(ctx, h, residual)

@@ -10,18 +10,22 @@ from .base import FeedForward, register_part
 
 @register_part("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
-    """down(act(gate(x)) * up(x)), no biases.  gate and up are kept as one matrix [2 * inner, hidden]."""
+    """down(act(gate(x), up(x))), no biases.  gate and up are kept as one matrix [2 * inner, hidden].  `activation`: one
+    of `ops.GATE_ACTIVATIONS` ("silu": silu(g) * u; "clamped_swish": g' = min(g, limit), u' = clamp(u, -limit, limit),
+    g' * sigmoid(1.702 g') * (u' + 1))."""
 
     graph_safe = True
 
     graph_safe_portions = True
 
     def __init__(self, hidden: int, inner: int, activation: str = "silu",
-                 tensors: tuple = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+                 tensors: tuple = ("gate_proj.weight", "up_proj.weight", "down_proj.weight"), limit: float = 0.0):
         if activation not in ops.GATE_ACTIVATIONS:     # refused when the part is built, not at the first step
             raise ValueError(f"Gated feed-forward with activation {activation!r} has no kernel; "
                              f"there are kernels for {sorted(ops.GATE_ACTIVATIONS)}.")
-        self.hidden, self.inner, self.activation = hidden, inner, activation
+        if activation == "clamped_swish" and not limit > 0:
+            raise ValueError(f"The clamped activation needs a positive limit, got {limit!r}.")
+        self.hidden, self.inner, self.activation, self.limit = hidden, inner, activation, float(limit)
         self.names = tuple(tensors)      # local names of the gate, up and down matrices
 
     def flops(self, tokens: int, pairs: int = 0) -> float:
@@ -53,7 +57,7 @@ class GatedMLP(FeedForward):
         if ctx.act_dtype == torch.float32 and self.fuse_input_norm_f32:
             act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
             if not ops.gate_up_silu_f32(self.w_gate_up, residual, act, activation=self.activation, norm_weight=fold.weight,
-                                        eps=fold.eps):
+                                        eps=fold.eps, limit=self.limit):
                 return False
             ops.gemm(act, self.w_down, residual, accumulate=True)
             return True
@@ -63,19 +67,23 @@ class GatedMLP(FeedForward):
             return False
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
         ops.gate_up_silu(self.w_gate_up, act, residual=residual, norm_weight=fold.weight, eps=fold.eps,
-                         activation=self.activation)
+                         activation=self.activation, limit=self.limit)
         ops.gemm(act, self.w_down, residual, accumulate=True)
         return True
 
-    def forward(self, ctx, h, residual):
+    def forward(self, ctx, h, residual, row_gate=None, row_gate_column: int = 0):
+        """`row_gate` (float32 [T, columns]): the token's output is multiplied by sigmoid(row_gate[t, row_gate_column]);
+        the factor goes onto the gated product, of which the output is a linear function."""
         T = h.shape[0]
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
-        if ctx.act_dtype == torch.bfloat16 and self._fused(T, False):
-            ops.gate_up_silu(self.w_gate_up, act, x=h, activation=self.activation)
-        elif ctx.act_dtype == torch.float32 and ops.gate_up_silu_f32(self.w_gate_up, h, act, activation=self.activation):
+        if row_gate is None and ctx.act_dtype == torch.bfloat16 and self._fused(T, False):
+            ops.gate_up_silu(self.w_gate_up, act, x=h, activation=self.activation, limit=self.limit)
+        elif row_gate is None and ctx.act_dtype == torch.float32 and ops.gate_up_silu_f32(
+                self.w_gate_up, h, act, activation=self.activation, limit=self.limit):
             pass
         else:
             gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)
             ops.gemm(h, self.w_gate_up, gu)
-            ops.silu_mul(gu, act, activation=self.activation)
+            ops.silu_mul(gu, act, activation=self.activation, limit=self.limit, row_gate=row_gate,
+                         row_gate_column=row_gate_column)
         ops.gemm(act, self.w_down, residual, accumulate=True)

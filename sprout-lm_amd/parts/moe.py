@@ -24,6 +24,13 @@ class RoutedExperts(FeedForward):
     hidden, inner, experts, top: sizes.  shared_inner: inner size of the shared expert (None: there is none).
     router_bias: whether the router has a bias.  `tensors`: local name patterns of an expert's gate, up and down
     matrices (`{e}` = the expert's number), of the router's weight and bias, and the prefix of the shared expert.
+
+    routing "scored_groups" is another rule of choice: scores s = the softmax over ALL router outputs; the choice goes by
+    s + correction (a tensor, `correction`) and only among the outputs of the `keep` best of `groups` equal groups of
+    neighbours (a group's worth is its largest such sum); the weights are the chosen outputs' s times `route_scale`, not
+    renormalised.  The last `identity` router outputs are experts without tensors that return their input.
+    activation / limit, shared_activation / shared_limit: see GatedMLP.  shared_gate: the local name of a [1, hidden]
+    tensor g; the shared expert's output is then multiplied by sigmoid(g . x), one number per token.
     """
 
     graph_safe = True
@@ -32,24 +39,50 @@ class RoutedExperts(FeedForward):
 
     def __init__(self, hidden: int, inner: int, experts: int, top: int, shared_inner: int | None = None,
                  router_bias: bool = True, activation: str = "silu",
-                 tensors: tuple = ("e{e}.gate", "e{e}.up", "e{e}.down", "router", "router.b", "shared.")):
-        if min(hidden, inner, experts, top) <= 0 or top > experts:
+                 tensors: tuple = ("e{e}.gate", "e{e}.up", "e{e}.down", "router", "router.b", "shared."),
+                 limit: float = 0.0, routing: str = "softmax_top", identity: int = 0, groups: int = 1, keep: int = 1,
+                 route_scale: float = 1.0, correction: str | None = None, shared_activation: str | None = None,
+                 shared_limit: float = 0.0, shared_gate: str | None = None):
+        if min(hidden, inner, experts, top) <= 0 or top > experts + identity or identity < 0:
             raise ConfigError(f"A routed feed-forward needs 0 < top <= experts and positive sizes, got top={top} "
                               f"experts={experts} inner={inner}.")
+        if routing not in ("softmax_top", "scored_groups"):
+            raise ConfigError(f"No routing rule {routing!r}; there are 'softmax_top' and 'scored_groups'.")
+        outputs = experts + identity
+        if routing == "softmax_top" and (identity or groups != 1 or correction or route_scale != 1.0):
+            raise ConfigError("Identity experts, groups, a correction and a scale belong to the rule 'scored_groups'.")
+        if routing == "scored_groups":
+            if groups <= 0 or outputs % groups or not 0 < keep <= groups or top > keep * (outputs // groups):
+                raise ConfigError(f"{outputs} router outputs do not form {groups} equal groups of which {keep} hold {top} choices.")
+            if outputs > 256:
+                raise ConfigError(f"The grouped rule of choice takes up to 256 router outputs, got {outputs}.")
+            if router_bias:
+                raise ConfigError("The grouped rule of choice has a correction on the scores, not a bias on the logits.")
+        if activation == "clamped_swish" and not limit > 0:
+            raise ConfigError(f"The clamped activation needs a positive limit, got {limit!r}.")
         if activation not in ops.GATE_ACTIVATIONS:
             raise ConfigError(f"Experts with activation {activation!r} have no kernel; there are kernels for "
                               f"{sorted(ops.GATE_ACTIVATIONS)}.")
         self.hidden, self.inner, self.experts, self.top = hidden, inner, experts, top
         self.router_bias, self.activation, self.names = router_bias, activation, tuple(tensors)
+        self.limit, self.routing, self.identity, self.groups, self.keep = float(limit), routing, identity, groups, keep
+        self.route_scale, self.correction, self.shared_gate = float(route_scale), correction, shared_gate
+        self.outputs = outputs
         prefix = self.names[5]
-        self.shared = None if not shared_inner else GatedMLP(hidden, shared_inner, activation,
-                                                             tensors=(prefix + "gate", prefix + "up", prefix + "down"))
+        try:
+            self.shared = None if not shared_inner else GatedMLP(hidden, shared_inner, shared_activation or activation,
+                                                                 tensors=(prefix + "gate", prefix + "up", prefix + "down"),
+                                                                 limit=shared_limit if shared_activation else limit)
+        except ValueError as error:
+            raise ConfigError(str(error)) from None
+        if shared_gate is not None and self.shared is None:
+            raise ConfigError("A gate on the shared expert needs a shared expert.")
 
     def subparts(self):
         return [self.shared] if self.shared is not None else []
 
     def flops(self, tokens: int, pairs: int = 0) -> float:
-        total = 2.0 * tokens * self.hidden * (self.experts + 3 * self.inner * self.top)
+        total = 2.0 * tokens * self.hidden * (self.outputs + 3 * self.inner * self.top)
         return total + (self.shared.flops(tokens) if self.shared is not None else 0.0)
 
     def tensors(self):
@@ -59,11 +92,15 @@ class RoutedExperts(FeedForward):
             out[gate.format(e=e)] = TensorSpec((self.inner, self.hidden))
             out[up.format(e=e)] = TensorSpec((self.inner, self.hidden))
             out[down.format(e=e)] = TensorSpec((self.hidden, self.inner))
-        out[router] = TensorSpec((self.experts, self.hidden))
+        out[router] = TensorSpec((self.outputs, self.hidden))
         if self.router_bias:
             out[bias] = TensorSpec((self.experts,), "vector")
+        if self.correction is not None:
+            out[self.correction] = TensorSpec((self.outputs,), "vector")
         if self.shared is not None:
             out.update(self.shared.tensors())
+        if self.shared_gate is not None:
+            out[self.shared_gate] = TensorSpec((1, self.hidden))
         return out
 
     def bind(self, tensors):
@@ -74,7 +111,10 @@ class RoutedExperts(FeedForward):
                                       for e in range(E)]).contiguous()
         self.w_down = torch.stack([tensors.pop(down.format(e=e)) for e in range(E)]).contiguous()
         self.w_router = tensors[router]
+        if self.shared_gate is not None:      # the gate's one row rides behind the router's: one product for both
+            self.w_router = torch.cat([self.w_router, tensors[self.shared_gate].reshape(1, self.hidden)], dim=0).contiguous()
         self.b_router = tensors[bias] if self.router_bias else None
+        self.w_correction = tensors[self.correction].to(torch.float32).contiguous() if self.correction is not None else None
         if self.shared is not None:
             self.shared.bind({name: tensors[name] for name in self.shared.tensors()})
         self.w = {}
@@ -82,7 +122,7 @@ class RoutedExperts(FeedForward):
     def forward(self, ctx, h, residual):
         T, E, top = h.shape[0], self.experts, self.top
         pairs = T * top
-        logits = ctx.buffer("router_logits", (T, E), torch.float32)
+        logits = ctx.buffer("router_logits", (T, self.w_router.shape[0]), torch.float32)
         ops.gemm(h, self.w_router, logits, bias=self.b_router)
         ids = ctx.buffer("expert_ids", (T, top), torch.int32)
         weights = ctx.buffer("expert_weights", (T, top), torch.float32)
@@ -91,12 +131,22 @@ class RoutedExperts(FeedForward):
         tile_rows = ops.group_tile_rows(ctx.act_dtype, pairs, E, self.hidden % 8 == 0 and self.inner % 8 == 0)
         tiles = ctx.buffer("expert_tiles", (3 * ops.route_max_tiles(pairs, E, tile_rows),), torch.int32)
         n_tiles = ctx.buffer("expert_tile_count", (1,), torch.int32)
-        ops.route(logits, ids, weights, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
+        if self.routing == "scored_groups":
+            ops.route_scored(logits, self.outputs, E, self.w_correction, self.groups, self.keep, self.route_scale, ids, weights,
+                             row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
+        else:
+            ops.route(logits, ids, weights, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
         act = ctx.buffer("expert_act", (pairs, self.inner), ctx.act_dtype)
         ops.expert_gate_up(h, self.w_gate_up, tiles, n_tiles, pair_of_row, top, act, activation=self.activation,
-                           tile_rows=tile_rows)
+                           tile_rows=tile_rows, limit=self.limit)
         out = ctx.buffer("expert_out", (pairs, self.hidden), torch.float32)
         ops.expert_down(act, self.w_down, tiles, n_tiles, out, tile_rows=tile_rows)
-        ops.route_combine(out, row_of_pair, weights, residual)
+        if self.identity:      # a pair routed to an identity output has no row of `out`: the sum takes the token's input
+            ops.route_combine_identity(out, row_of_pair, ids, weights, h, E, residual)
+        else:
+            ops.route_combine(out, row_of_pair, weights, residual)
         if self.shared is not None:
-            self.shared.forward(ctx, h, residual)
+            if self.shared_gate is not None:
+                self.shared.forward(ctx, h, residual, row_gate=logits, row_gate_column=self.outputs)
+            else:
+                self.shared.forward(ctx, h, residual)

@@ -65,6 +65,9 @@ def _register_builtin():
     from .config.megozen import MegozenConfig
     from .models.megozen import build_megozen
     register_architecture(MegozenConfig.architecture, MegozenConfig, build_megozen)
+    from .config.bogilix import BogilixConfig
+    from .models.bogilix import build_bogilix
+    register_architecture(BogilixConfig.architecture, BogilixConfig, build_bogilix)
 
 
 _register_builtin()
