@@ -181,8 +181,8 @@ class BogilixConfig(ModelConfig):
             mlp = _section(entry, "mlp", where, optional=True)
             layers.append(BogilixLayer(kind, mixer, FeedForwardSizes.parse(mlp, where + "mlp.") if mlp is not None else None))
         mixing = [layer.mixer for layer in layers if layer.mixer.v_mix]
-        if any((m.kv_heads, m.vdim) != (mixing[0].kv_heads, mixing[0].vdim) for m in mixing):
-            raise ConfigError(_WHAT + "layers that blend their values with the first such layer's must have its kv_heads and vdim.")
+        if any(m.kv_heads * m.vdim != mixing[0].kv_heads * mixing[0].vdim for m in mixing):
+            raise ConfigError(_WHAT + "layers that blend their values with the first such layer's must have as many value numbers a token.")
         return cls(vocab, width, eps, tuple(layers))
 
     def to_dict(self) -> dict:

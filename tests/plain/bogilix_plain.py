@@ -183,7 +183,7 @@ def _values(w, pre, m, v, shared, store):
     if "first" not in shared:
         shared["first"] = v
         return v
-    return store(blend_values(v, shared["first"], np.asarray(w[pre + "vmix"]).reshape(())))
+    return store(blend_values(v, shared["first"].reshape(v.shape), np.asarray(w[pre + "vmix"]).reshape(())))
 
 
 # ---------------------------------------------------------------------------------------------- feed-forwards

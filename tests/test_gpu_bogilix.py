@@ -1,0 +1,659 @@
+"""Bogilix on the GPU: every mechanism alone against its plain function, then whole models cut into steps in
+different ways, then generation through the engine's entry point and scheduler."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import bogilix_helpers as BH
+from tests import traces
+from tests.plain import bogilix_plain as B
+from tests.test_gpu_megozen import Harness, dev
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def rounded(x, dtype):
+    return B.bf16_round(x) if dtype == torch.bfloat16 else np.asarray(x, np.float32)
+
+
+def store_of(dtype):
+    return B.bf16_round if dtype == torch.bfloat16 else B.f32
+
+
+def close(got, want, dtype, what, f32=2e-5, bf16=2e-2):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    bound = (f32 if dtype == torch.float32 else bf16) * max(1.0, float(np.abs(want).max()))
+    err = float(np.abs(got - want).max())
+    assert err <= bound, f"{what}: off by {err:.3e} (bound {bound:.1e})"
+
+
+# ---------------------------------------------------------------------------------------------- mechanisms alone
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [24, 100, 256, 4100])
+def test_layer_norm_with_bias(dtype, H):
+    """Rows with a mean far from zero, all rows and gathered rows, a bias, and two norms of one input in one pass."""
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.parts import make_part
+    rng = np.random.default_rng(H)
+    part = make_part("norm", "layernorm", size=H, eps=1e-5, tensor="norm1", bias="norm1.b")
+    assert list(part.tensors()) == ["norm1", "norm1.b"]
+    x = (rng.normal(0, 1, (9, H)) + 40.0).astype(np.float32)
+    w, b = rounded(1 + rng.normal(0, 0.1, H), dtype), rounded(rng.normal(0, 0.5, H), dtype)
+    part.bind({"norm1": dev(w, dtype), "norm1.b": dev(b, dtype)})
+    out = torch.empty(9, H, dtype=dtype, device=DEV)
+    part.forward(None, dev(x), out)
+    close(out.float().cpu().numpy(), B.layer_norm(x, w, b, 1e-5), dtype, "all rows")
+    rows = [7, 0, 3]
+    out = torch.empty(3, H, dtype=dtype, device=DEV)
+    part.forward(None, dev(x), out, rows=torch.tensor(rows, dtype=torch.int32, device=DEV))
+    close(out.float().cpu().numpy(), B.layer_norm(x[rows], w, b, 1e-5), dtype, "gathered rows")
+    w2, b2 = rounded(1 + rng.normal(0, 0.1, H), dtype), rounded(rng.normal(0, 0.5, H), dtype)
+    o1, o2 = torch.empty(9, H, dtype=dtype, device=DEV), torch.empty(9, H, dtype=dtype, device=DEV)
+    ops.layernorm(dev(x), dev(w, dtype), 1e-5, o1, None, dev(w2, dtype), o2, bias=dev(b, dtype), bias2=dev(b2, dtype))
+    close(o1.float().cpu().numpy(), B.layer_norm(x, w, b, 1e-5), dtype, "first of two")
+    close(o2.float().cpu().numpy(), B.layer_norm(x, w2, b2, 1e-5), dtype, "second of two")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,dim,vdim,rot,norm", [(3, 3, 20, 6, 8, False), (6, 2, 12, 10, 0, True), (4, 1, 64, 32, 64, False),
+                                                        (8, 1, 48, 64, 0, True), (2, 2, 16, 16, 6, True)])
+def test_prepare_norms_turns_blends_and_writes_the_cache(dtype, nq, nkv, dim, vdim, rot, norm):
+    """Whole-row norms, the rotation of a head's first numbers at positions up to a million, the blend with kept values,
+    queries at the padded width with zeros behind, and keys and values where the slot mapping says (a negative slot
+    writes nothing; a page written before keeps no stale number behind the head)."""
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.parts.sink_attention import padded_width
+    rng = np.random.default_rng(nq * 100 + dim)
+    T, page, pages, eps, base = 7, 4, 6, 1e-5, 250.0
+    W = padded_width(dim, vdim)
+    # (the bfloat16 path takes its angles in float32: off by position * 6e-8, which its tolerance holds up to some 10^4)
+    positions = np.asarray([0, 1, 5, 63, 64, 1000, 1_000_000 if dtype == torch.float32 else 20_000])
+    cols = (nq + nkv) * dim + nkv * vdim
+    proj = rounded(rng.normal(0, 1, (T, cols)), dtype)
+    qn, kn = rounded(1 + rng.normal(0, 0.1, nq * dim), dtype), rounded(1 + rng.normal(0, 0.1, nkv * dim), dtype)
+    first = rounded(rng.normal(0, 1, (T, nkv * vdim)), dtype)
+    lam = float(rounded(np.asarray([0.3]), dtype)[0])
+    store = store_of(dtype)
+    q = proj[:, :nq * dim].astype(np.float64)
+    k = proj[:, nq * dim:(nq + nkv) * dim].astype(np.float64)
+    v = proj[:, (nq + nkv) * dim:].astype(np.float64)
+    if norm:
+        q, k = store(B.rms_norm(q, qn, eps)), store(B.rms_norm(k, kn, eps))
+    q = store(B.turn_halves(q.reshape(T, nq, dim), positions, rot, base))
+    k = store(B.turn_halves(k.reshape(T, nkv, dim), positions, rot, base))
+    inv = base ** (-2.0 * np.arange(rot // 2, dtype=np.float64) / max(rot, 1))
+    inv32 = inv.astype(np.float32)
+    tail = (inv - inv32.astype(np.float64)).astype(np.float32)
+    slots = np.asarray([9, 2, -1, 11, 0, 23, 5], dtype=np.int32)
+    for mode in ("plain", "keep", "blend"):
+        k_pool = torch.full((pages, nkv, page, W), 7.0, dtype=dtype, device=DEV)
+        v_pool = torch.full((pages, nkv, W, page), 7.0, dtype=dtype, device=DEV)
+        q_out = torch.full((T, nq * W), 7.0, dtype=dtype, device=DEV)
+        kept = dev(first, dtype).clone()
+        ops.qkv_prepare(dev(proj, dtype), nq, nkv, dim, vdim, W, q_out, positions=dev(positions, torch.int32),
+                        inv_freq=dev(inv32) if rot else None, inv_freq_tail=dev(tail) if rot and dtype == torch.float32 else None,
+                        rotary_dim=rot, q_norm=dev(qn, dtype) if norm else None, k_norm=dev(kn, dtype) if norm else None, eps=eps,
+                        blend=dev(np.asarray([lam]), dtype) if mode == "blend" else None,
+                        first=kept if mode != "plain" else None, keep_first=mode == "keep",
+                        slot_mapping=dev(slots, torch.int32), k_pool=k_pool, v_pool=v_pool)
+        want_v = store(B.blend_values(v, first, lam)) if mode == "blend" else v
+        got_q = q_out.float().cpu().numpy().reshape(T, nq, W)
+        close(got_q[:, :, :dim], q, dtype, f"{mode}: queries", f32=3e-6, bf16=1e-2)
+        assert not got_q[:, :, dim:].any(), "numbers behind a query head must be zero"
+        if mode == "keep":
+            close(kept.float().cpu().numpy(), v, dtype, "kept values", f32=0, bf16=0)
+        kp, vp = k_pool.float().cpu().numpy(), v_pool.float().cpu().numpy()
+        for t, slot in enumerate(slots):
+            if slot < 0:
+                continue
+            close(kp[slot // page, :, slot % page, :dim], k[t], dtype, f"{mode}: key of token {t}", f32=3e-6, bf16=1e-2)
+            assert not kp[slot // page, :, slot % page, dim:].any() and not vp[slot // page, :, vdim:, slot % page].any()
+            close(vp[slot // page, :, :vdim, slot % page], want_v[t].reshape(nkv, vdim), dtype, f"{mode}: value of token {t}", f32=1e-6, bf16=1e-2)
+        untouched = [s for s in range(pages * page) if s not in set(slots.tolist())]
+        assert all((kp[s // page, :, s % page] == 7.0).all() for s in untouched), "a slot nobody named was written"
+
+
+def attention_case(rng, dtype, nq, nkv, W, dim, vdim, lengths, flagged):
+    """Queries, keys, values of sequences of `lengths`; `flagged` [(sequence, query, key)]: that query and key are
+    scaled so that their score towers over the others of the row, and the key's value is far from the rest."""
+    seqs = []
+    for n in lengths:
+        q = rng.normal(0, 1, (n, nq, dim))
+        k = rng.normal(0, 1, (n, nkv, dim))
+        v = rng.normal(0, 1, (n, nkv, vdim))
+        seqs.append([q, k, v])
+    for s, i, j in flagged:
+        q, k, v = seqs[s]
+        direction = rng.normal(0, 1, dim)
+        direction /= np.linalg.norm(direction)
+        q[i] = 6.0 * direction
+        k[j] = 6.0 * direction
+        v[j] += 8.0
+    return [[rounded(a, dtype).astype(np.float64) for a in seq] for seq in seqs]
+
+
+def run_attention(dtype, seqs, cuts, nq, nkv, W, dim, vdim, scale, chunk, cap, sinks, page, kind=0, window=None):
+    """The attention entry point over a paged cache filled step by step; `cuts`: per step [(sequence, tokens)].
+    Returns per sequence the outputs [n, nq, vdim] (and checks that the padded columns stay zero)."""
+    from sprout_lm_amd import ops
+    from sprout_lm_amd.cache.spec import PagedKVSpec
+    reach = min([n for n in (chunk, window) if n]) if (chunk or window) else None
+    h = Harness([PagedKVSpec(nkv, W, reach)], dtype, page=page, pages=256)
+    live = [h.cache.create() for _ in seqs]
+    outs = [np.zeros((len(s[0]), nq, vdim)) for s in seqs]
+    for step in cuts:
+        batch = [(live[s], [0] * n) for s, n in step]
+        ctx, entries = h.context(batch)
+        view = h.view(ctx, 0)
+        T = sum(n for _, n in step)
+        q = np.zeros((T, nq, W), np.float32)
+        at = 0
+        slot_map = ctx.group_slots[0].cpu().numpy() if hasattr(ctx.group_slots[0], "cpu") else ctx.group_slots[0]
+        kp, vp = view.k, view.v
+        for s, n in step:
+            lo = live[s].length
+            q[at:at + n, :, :dim] = seqs[s][0][lo:lo + n]
+            kk = np.zeros((n, nkv, W), np.float32); kk[:, :, :dim] = seqs[s][1][lo:lo + n]
+            vv = np.zeros((n, nkv, W), np.float32); vv[:, :, :vdim] = seqs[s][2][lo:lo + n]
+            for i in range(n):
+                slot = int(slot_map[at + i])
+                kp[slot // page, :, slot % page, :] = dev(kk[i], dtype)
+                vp[slot // page, :, :, slot % page] = dev(vv[i], dtype)
+            at += n
+        out = torch.zeros(T, nq * W, dtype=dtype, device=DEV)
+        ops.attention(dev(q.reshape(T, -1), dtype), nq * W, kp, vp, view.block_tables, ctx.attention, out, nq, nkv, W, window, scale,
+                      kind=kind, scores="capped" if cap else "scaled_dot", softcap=cap or 0.0,
+                      sinks=dev(sinks) if sinks is not None else None, mask_chunk=chunk)
+        got = out.float().cpu().numpy().reshape(T, nq, W)
+        assert not got[:, :, vdim:].any()
+        at = 0
+        for s, n in step:
+            lo = live[s].length
+            outs[s][lo:lo + n] = got[at:at + n, :, :vdim]
+            at += n
+        h.commit(entries)
+    return outs
+
+
+ATT_SHAPES = [  # nq, nkv, dim, vdim, chunk, cap, page
+    (8, 1, 48, 64, 64, 50.0, 16),     # keys narrower than values, matrix-core width 64
+    (4, 2, 64, 32, 33, None, 8),      # keys wider, blocks that are no multiple of a page
+    (32, 1, 16, 32, 16, 4.0, 16),     # more heads than a block of the one-query kernel holds
+    (3, 3, 20, 6, 5, None, 4),        # a width only the general kernel takes
+    (6, 2, 12, 10, 300, 7.0, 16),     # blocks longer than a chunk of the one-query kernels
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", ATT_SHAPES)
+@pytest.mark.parametrize("kind", [0, 1])
+def test_attention_blocks_cap_and_sinks(dtype, shape, kind):
+    """Prompts in portions and single queries over keys in pages: a flagged key just inside a query's block (its first
+    position), just outside (the last position of the block before), far back in the block, at a page's first and last
+    place; sinks from far below the scores to far above them; capped scores where the flagged score exceeds the cap
+    many times over.  kind 1 is the float32-arithmetic kernel, 0 the engine's choice (matrix cores where sizes allow)."""
+    from sprout_lm_amd.parts.sink_attention import padded_width
+    nq, nkv, dim, vdim, chunk, cap, page = shape
+    W = padded_width(dim, vdim)
+    rng = np.random.default_rng(dim * 7 + chunk)
+    lengths = [max(3 * chunk + 7, 40), 2 * chunk + 1, 1, 700 if chunk == 300 else 150]
+    flagged = []
+    for s, n in enumerate(lengths):
+        for i in range(n):
+            lo = i - i % chunk
+            if i % 11 == 3 and i > 0:
+                flagged.append((s, i, lo))                      # the block's first position: just inside
+            elif i % 11 == 5 and lo > 0:
+                flagged.append((s, i, lo - 1))                  # the block before's last: just outside
+            elif i % 11 == 8 and i - lo > 2:
+                flagged.append((s, i, lo + (i - lo) // 2))      # somewhere in between
+    # a query flagged twice would lose its first flag: keep one per query, and never reuse a key
+    seen_q, seen_k, kept = set(), set(), []
+    for s, i, j in flagged:
+        if (s, i) not in seen_q and (s, j) not in seen_k and (s, j) not in seen_q and (s, i) not in seen_k:
+            seen_q.add((s, i)); seen_k.add((s, j)); kept.append((s, i, j))
+    seqs = attention_case(rng, dtype, nq, nkv, W, dim, vdim, lengths, kept)
+    sinks = np.linspace(-30.0, 12.0, nq).astype(np.float32)
+    scale = 0.35
+    # step 1: most of every prompt in portions beside each other; then tokens one by one (all sequences in a step)
+    cuts = []
+    fed = [0] * len(lengths)
+    tails = [min(n - 1, 2 * chunk + 3 if chunk < 100 else 40) for n in lengths]
+    sizes = [37, 2, 16, 64, 3, 129]
+    i = 0
+    while any(fed[s] < lengths[s] - tails[s] for s in range(len(lengths))):
+        step = []
+        for s in range(len(lengths)):
+            left = lengths[s] - tails[s] - fed[s]
+            if left > 0:
+                n = min(sizes[(i + s) % len(sizes)], left)
+                step.append((s, n)); fed[s] += n
+        cuts.append(step); i += 1
+    while any(fed[s] < lengths[s] for s in range(len(lengths))):
+        step = [(s, 1) for s in range(len(lengths)) if fed[s] < lengths[s]]
+        for s, _ in step:
+            fed[s] += 1
+        cuts.append(step)
+    outs = run_attention(dtype, seqs, cuts, nq, nkv, W, dim, vdim, scale, chunk, cap, sinks, page, kind=kind)
+    for s, (q, k, v) in enumerate(seqs):
+        want = B.attend(q, k, v, nq, nkv, scale, chunk, sinks, cap, store=lambda a: a).reshape(len(q), nq, vdim)
+        close(outs[s], want, dtype, f"sequence {s}", f32=2e-5, bf16=2.5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_sink_alone_and_window_with_blocks(dtype):
+    """A sink far above every score leaves (almost) nothing of the values; one far below changes nothing; a window and
+    blocks together let a query see what both allow."""
+    nq, nkv, dim, vdim, W, page = 4, 2, 32, 32, 32, 8
+    rng = np.random.default_rng(5)
+    seqs = attention_case(rng, dtype, nq, nkv, W, dim, vdim, [90], [])
+    cuts = [[(0, 50)]] + [[(0, 1)]] * 40
+    high = run_attention(dtype, seqs, cuts, nq, nkv, W, dim, vdim, 0.2, 40, None, np.full(nq, 60.0, np.float32), page)[0]
+    assert np.abs(high).max() < 1e-6
+    low = run_attention(dtype, seqs, cuts, nq, nkv, W, dim, vdim, 0.2, 40, None, np.full(nq, -80.0, np.float32), page)[0]
+    none = run_attention(dtype, seqs, cuts, nq, nkv, W, dim, vdim, 0.2, 40, None, None, page)[0]
+    close(low, none, dtype, "a sink far below", f32=1e-6, bf16=1e-6)
+    both = run_attention(dtype, seqs, cuts, nq, nkv, W, dim, vdim, 0.2, 40, None, None, page, window=7)[0]
+    q, k, v = seqs[0]
+    want = np.zeros_like(both)
+    for i in range(90):
+        lo = max(i - 6, i - i % 40)
+        for h in range(nq):
+            s = (k[lo:i + 1, h // 2] @ q[i, h]) * 0.2
+            p = np.exp(s - s.max()); p /= p.sum()
+            want[i, h] = p @ v[lo:i + 1, h // 2]
+    close(both, want, dtype, "window and blocks", f32=2e-5, bf16=2.5e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I,K", [(1, 24, 40), (9, 96, 64), (40, 64, 128), (130, 96, 64), (300, 128, 256), (16, 28, 100)])
+def test_clamped_gate_and_row_gate(dtype, T, I, K):
+    """The clamped activation on every path a gated product takes (the element-wise kernel, the kernels that fold it
+    into the product for few tokens and for many), with gate and up values beyond the limit on both sides, and the
+    sigmoid of one number per token on a row."""
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(T + I)
+    limit = 0.75
+    x = rounded(rng.normal(0, 1, (T, K)), dtype)
+    w = rounded(rng.normal(0, 0.3, (2 * I, K)), dtype)
+    store = store_of(dtype)
+    g, u = store(B.linear(x, w[:I])), store(B.linear(x, w[I:]))
+    assert (g > limit).any() and (u > limit).any() and (u < -limit).any()
+    gc, uc = np.minimum(g, limit), np.clip(u, -limit, limit)
+    want = gc * B.sigmoid(1.702 * gc) * (uc + 1.0)
+    gu = dev(np.concatenate([g, u], axis=1), dtype)
+    out = torch.empty(T, I, dtype=dtype, device=DEV)
+    ops.silu_mul(gu, out, activation="clamped_swish", limit=limit)
+    close(out.float().cpu().numpy(), want, dtype, "element-wise", f32=2e-6, bf16=1e-2)
+    gate = rng.normal(0, 2, (T, 3)).astype(np.float32)
+    ops.silu_mul(gu, out, activation="clamped_swish", limit=limit, row_gate=dev(gate), row_gate_column=2)
+    close(out.float().cpu().numpy(), want * B.sigmoid(gate[:, 2:3]), dtype, "with a row gate", f32=2e-6, bf16=1e-2)
+    from sprout_lm_amd.parts import make_part
+    part = make_part("feed_forward", "gated_mlp", hidden=K, inner=I, activation="clamped_swish", limit=limit, tensors=("gate", "up", "down"))
+    down = rounded(rng.normal(0, 0.2, (K, I)), dtype)
+    part.bind({"gate": dev(w[:I], dtype), "up": dev(w[I:], dtype), "down": dev(down, dtype)})
+    from sprout_lm_amd.engine.batch import StepContext, Workspace
+    ctx = StepContext(Workspace(DEV), dtype, 0)
+    residual = torch.zeros(T, K, dtype=torch.float32, device=DEV)
+    part.forward(ctx, dev(x, dtype), residual)
+    close(residual.cpu().numpy(), B.linear(store(want), down), dtype, "the part", f32=2e-5, bf16=2e-2)
+
+
+def test_scored_routing_choice_ties_groups_and_identity():
+    """The grouped rule against the plain one on random logits; then crafted rows: a correction that turns the choice
+    but not the weights, negative sums (a shut group must not win with a 0), ties (the lower index), a group whose best
+    is high but whose others are low, identity outputs that get rows behind the experts' and no tiles."""
+    from sprout_lm_amd import ops
+    rng = np.random.default_rng(3)
+    for outputs, real, top, groups, keep, T in ((10, 8, 2, 2, 1, 300), (6, 5, 3, 3, 2, 50), (9, 9, 4, 1, 1, 700), (12, 7, 6, 4, 2, 40),
+                                                (200, 190, 8, 10, 3, 20), (4, 3, 4, 2, 2, 9), (5, 5, 1, 5, 1, 33)):
+        z = rng.normal(0, 2, (T, outputs + 1)).astype(np.float32)          # a further column rides behind, as a gate's would
+        corr = rng.normal(0, 0.3, outputs).astype(np.float32)
+        if outputs == 10:
+            corr -= 2.0                                                    # every sum negative
+            z[5, :outputs] = 0.0                                           # all equal: the lowest indices of the best group
+            z[6, :outputs] = [5, 0, 0, 0, 0, 4.9, 4.9, 4.9, 4.9, 4.9]      # one high head in group 0 beats a strong group 1
+        want_ids, want_w = B.route(z[:, :outputs], corr, top, groups, keep, 1.7)
+        tile_rows = 64
+        ids = torch.empty(T, top, dtype=torch.int32, device=DEV)
+        w = torch.empty(T, top, dtype=torch.float32, device=DEV)
+        pairs = T * top
+        row_of_pair = torch.empty(pairs, dtype=torch.int32, device=DEV)
+        pair_of_row = torch.empty(pairs, dtype=torch.int32, device=DEV)
+        tiles = torch.full((3 * ops.route_max_tiles(pairs, real, tile_rows),), -1, dtype=torch.int32, device=DEV)
+        n_tiles = torch.zeros(1, dtype=torch.int32, device=DEV)
+        ops.route_scored(dev(z), outputs, real, dev(corr), groups, keep, 1.7, ids, w, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
+        got_ids = ids.cpu().numpy()
+        # float32 scores against float64: a choice may differ only where the two sums are closer than rounding
+        e = np.exp(z[:, :outputs].astype(np.float64) - z[:, :outputs].max(-1, keepdims=True)); s = e / e.sum(-1, keepdims=True)
+        for t in range(T):
+            if list(got_ids[t]) != list(want_ids[t]):
+                c = s[t] + corr
+                assert sorted(got_ids[t]) == sorted(want_ids[t]) or np.abs(np.sort(c[got_ids[t]]) - np.sort(c[want_ids[t]])).max() < 1e-6, (outputs, t)
+            else:
+                np.testing.assert_allclose(w.cpu().numpy()[t], want_w[t], rtol=2e-5, atol=1e-7)
+        n = int(n_tiles.item())
+        tl = tiles.cpu().numpy()[:3 * n].reshape(n, 3)
+        assert (tl[:, 0] < real).all() and (tl[:, 2] <= tile_rows).all() and (tl[:, 2] > 0).all()
+        rp, pr = row_of_pair.cpu().numpy(), pair_of_row.cpu().numpy()
+        assert sorted(rp.tolist()) == list(range(pairs)) and (pr[rp] == np.arange(pairs)).all()
+        flat = got_ids.reshape(-1)
+        assert (np.diff(flat[pr]) >= 0).all(), "rows are ordered by expert"
+        covered = sum(int(r) for r in tl[:, 2])
+        assert covered == int((flat < real).sum())
+
+
+def expert_weights(rng, hidden, f, dtype):
+    w = {}
+    E, I = f["router"]["experts"], f["router"].get("identity", 0)
+    for e in range(E):
+        w[f"e{e}.gate"] = rounded(rng.normal(0, 0.2, (f["expert"]["ff"], hidden)), dtype)
+        w[f"e{e}.up"] = rounded(rng.normal(0, 0.2, (f["expert"]["ff"], hidden)), dtype)
+        w[f"e{e}.down"] = rounded(rng.normal(0, 0.2, (hidden, f["expert"]["ff"])), dtype)
+    w["router"] = rounded(rng.normal(0, 0.5, (E + I, hidden)), dtype)
+    w["correction"] = rounded(rng.normal(0, 0.05, E + I), dtype)
+    if f.get("shared"):
+        n = f["shared"]["ff"]
+        w["shared.gate"] = rounded(rng.normal(0, 0.2, (n, hidden)), dtype)
+        w["shared.up"] = rounded(rng.normal(0, 0.2, (n, hidden)), dtype)
+        w["shared.down"] = rounded(rng.normal(0, 0.2, (hidden, n)), dtype)
+        w["shared.sg"] = rounded(rng.normal(0, 0.5, (1, hidden)), dtype)
+    return w
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,f", [(40, BH.moe(5, 1, 3, 3, 2, 1.5, 28, 0.8, shared=(20, 1.2))),
+                                      (64, BH.moe(4, 0, 4, 1, 1, 0.9, 24, 0.5)),
+                                      (128, BH.moe(6, 2, 8, 4, 4, 2.0, 64, 1.0, shared=(64, 0.6)))])
+@pytest.mark.parametrize("T", [1, 7, 150, 1100])
+def test_routed_experts_part_with_grouped_choice(dtype, hidden, f, T):
+    """The routed feed-forward alone, from one token (tiles of 16 rows) to 1,100 (tiles of 256), with identity experts
+    and the gated shared expert.  bfloat16 is held to the cases in which every output is chosen."""
+    from sprout_lm_amd.parts import make_part
+    r = f["router"]
+    if dtype == torch.bfloat16 and r["top"] != r["experts"] + r["identity"]:
+        pytest.skip("a rounding may flip a choice")
+    rng = np.random.default_rng(hidden + T)
+    w = expert_weights(rng, hidden, f, dtype)
+    part = make_part("feed_forward", "routed_experts", hidden=hidden, inner=f["expert"]["ff"], experts=r["experts"], top=r["top"],
+                     router_bias=False, activation="clamped_swish", limit=f["expert"]["limit"], routing="scored_groups",
+                     identity=r["identity"], groups=r["groups"]["count"], keep=r["groups"]["keep"], route_scale=r["scale"],
+                     correction="correction", shared_inner=f["shared"]["ff"] if f.get("shared") else None,
+                     shared_activation="clamped_swish" if f.get("shared") else None,
+                     shared_limit=f["shared"]["limit"] if f.get("shared") else 0.0,
+                     shared_gate="shared.sg" if f.get("shared") else None)
+    assert sorted(part.tensors()) == sorted(w)
+    part.bind({n: dev(a, dtype) for n, a in w.items()})
+    x = rounded(rng.normal(0, 1, (T, hidden)), dtype)
+    from sprout_lm_amd.engine.batch import StepContext, Workspace
+    ctx = StepContext(Workspace(DEV), dtype, 0)
+    residual = torch.zeros(T, hidden, dtype=torch.float32, device=DEV)
+    part.forward(ctx, dev(x, dtype), residual)
+    want = B.routed_ff({("" + n): a for n, a in w.items()}, "", f, x, store_of(dtype))
+    close(residual.cpu().numpy(), want, dtype, "routed feed-forward", f32=3e-5, bf16=3e-2)
+
+
+# ---------------------------------------------------------------------------------------------- whole models
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = str(tmp_path_factory.mktemp("bogilix"))
+    return {name: BH.make_folder(root, name) for name in BH.CONFIGS}
+
+
+def requests_for(name, lengths, seed=100):
+    vocab = BH.CONFIGS[name]["vocab"]
+    return {f"r{i}": BH.random_tokens(vocab, n, seed + i) for i, n in enumerate(lengths)}
+
+
+def replay(folder, name, dtype, trace, max_tokens, page=None, slots=4, reused=None):
+    """The engine's trace session on a pool of `max_tokens`; per step the logits rows."""
+    from sprout_lm_amd.engine import ModelRunner
+    from sprout_lm_amd.engine.trace import TraceSession
+    page = page or BH.PAGE[name]
+    runner = ModelRunner.from_folder(folder, dtype, block_size=page, num_blocks=-(-max_tokens // page), max_sequences=slots,
+                                     prefix_caching=False)
+    session = TraceSession(runner)
+    out, owners = [], {}
+    for record in trace.steps:
+        logits = session.run_step(record)
+        out.append(None if logits is None or not logits.shape[0] else logits.cpu().numpy().copy())
+        for rid, seq in session.live.items():
+            for g, blocks in enumerate(seq.blocks):
+                for page_id in blocks:
+                    if page_id >= 0 and rid not in owners.setdefault((g, page_id), []):
+                        owners[(g, page_id)].append(rid)
+    if reused is not None:
+        reused["pages"] = sum(len(r) > 1 for r in owners.values())
+    assert all(free == total for free, total in zip(runner.cache.free_pages(), [g.pool.num_pages for g in runner.cache.groups]))
+    assert not session.live
+    return out
+
+
+def check(folder, dtype, requests, trace, results):
+    worst = 0.0
+    for step, (rows, got) in enumerate(zip(trace.expected, results)):
+        if not rows:
+            assert got is None
+            continue
+        assert got.shape[0] == len(rows)
+        for i, (rid, pos) in enumerate(rows):
+            want = BH.plain_logits(folder, dtype, requests[rid])[pos]
+            err = float(np.abs(got[i] - want).max())
+            worst = max(worst, err)
+            assert err <= BH.tolerance(dtype, want), f"step {step} request {rid} position {pos}: error {err:.3e}"
+    return worst
+
+
+LENGTHS = {"odd": [1, 2, 21, 70, 45, 97], "general": [1, 9, 40, 97, 150, 33, 2, 75], "all_chosen": [9, 40, 97, 33, 130],
+           "dense": [2, 70, 97, 33, 64, 120]}
+CASES = [(n, "float32") for n in BH.CONFIGS] + [("all_chosen", "bfloat16"), ("dense", "bfloat16")]
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+@pytest.mark.parametrize("family", ["whole", "tail", "portions", "mixed"])
+def test_replay_family(folders, name, dtype, family):
+    """Whole prompts; a prompt and its last 48 tokens one by one (blocks of 1 to 70 positions end among the decoded
+    tokens); portions down to two tokens; four live requests in a pool that holds no more, so that pages are used again."""
+    requests = requests_for(name, LENGTHS[name])
+    roomy = 4 * 64 * (1 + max(LENGTHS[name]) // 64)
+    if family == "whole":
+        trace, pool = traces.whole(requests), roomy
+    elif family == "tail":
+        trace, pool = traces.tail_decoded(requests, tail=48), roomy
+    elif family == "portions":
+        trace, pool = traces.portions(requests), roomy
+    else:
+        trace = traces.mixed(requests, seed=7)
+        pool = sum(sorted(-(-len(t) // 64) * 64 for t in requests.values())[-4:])
+    reused = {}
+    results = replay(folders[name], name, dtype, trace, pool, reused=reused)
+    if family == "mixed":
+        assert reused["pages"] >= 2, f"no page was used again: {reused}"
+    worst = check(folders[name], dtype, requests, trace, results)
+    print(f"{family} {name} {dtype}: {len(trace.steps)} steps, worst error {worst:.3e}")
+
+
+@pytest.mark.parametrize("name,page", [("general", 12), ("odd", 4), ("dense", 64)])
+def test_replay_with_other_page_sizes(folders, name, page):
+    requests = requests_for(name, LENGTHS[name], seed=300)
+    trace = traces.mixed(requests, seed=11)
+    pool = sum(sorted(-(-len(t) // 64) * 64 for t in requests.values())[-4:])
+    results = replay(folders[name], name, "float32", trace, pool, page=page)
+    check(folders[name], "float32", requests, trace, results)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_cuts_agree_with_each_other(folders, dtype):
+    """Whole, token-by-token and portioned replays give the same logits beyond rounding."""
+    name = "all_chosen"
+    requests = requests_for(name, [90])
+    rows_of = {}
+    for family, trace in (("whole", traces.whole(requests)), ("tail", traces.tail_decoded(requests, tail=89)),
+                          ("portions", traces.portions(requests))):
+        results = replay(folders[name], name, dtype, trace, 256)
+        rows_of[family] = {key: got[i] for expect, got in zip(trace.expected, results) for i, key in enumerate(expect)}
+    bound = 1e-5 if dtype == "float32" else 3e-2
+    for key, row in rows_of["whole"].items():
+        for other in ("tail", "portions"):
+            if key in rows_of[other]:
+                assert np.abs(row - rows_of[other][key]).max() <= bound * max(1.0, np.abs(row).max()), (key, other)
+
+
+def test_first_tokens_and_long_decoding(folders):
+    """Positions 0, 1, 2, ... fed one by one from the very first token, 260 in a row, past every block's edge."""
+    from sprout_lm_amd.engine import ModelRunner, StepEntry
+    for name, dtype in (("general", "float32"), ("dense", "bfloat16")):
+        tokens = BH.random_tokens(BH.CONFIGS[name]["vocab"], 260, 9)
+        runner = ModelRunner.from_folder(folders[name], dtype, block_size=8, num_blocks=40, max_sequences=2,
+                                         prefix_caching=False)
+        seq = runner.cache.create()
+        want = BH.plain_logits(folders[name], dtype, tokens)
+        for p, token in enumerate(tokens):
+            assert runner.cache.reserve(seq, p + 1)
+            got = runner.step([StepEntry(seq, [token], [0])]).cpu().numpy()[0]
+            assert np.abs(got - want[p]).max() <= BH.tolerance(dtype, want[p]), f"{name} {dtype} position {p}"
+        seq.release()
+
+
+def test_trace_run_program(folders, tmp_path):
+    """bin/trace_run as a user runs it, on a model it picks by the folder's config.json."""
+    name, dtype = "general", "float32"
+    requests = requests_for(name, [33, 70, 20, 64, 45])
+    trace = traces.mixed(requests, seed=3)
+    pool = sum(sorted(-(-len(t) // 64) * 64 for t in requests.values())[-4:])
+    out = tmp_path / "logits"
+    proc = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", folders[name],
+                             "--dtype", dtype, "--out", str(out), "--max-tokens", str(pool), "--max-sequences", "4"],
+                            stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True, bufsize=1)
+    try:
+        for record in trace.steps:
+            proc.stdin.write(json.dumps(record) + "\n")
+            proc.stdin.flush()
+            assert proc.stdout.readline().strip() == f"done {record['step']}"
+        proc.stdin.close()
+        assert proc.wait(timeout=60) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    vocab = BH.CONFIGS[name]["vocab"]
+    results = [np.fromfile(out / f"{r['step']}.f32", dtype="<f4").reshape(len(rows), vocab) if rows else None
+               for r, rows in zip(trace.steps, trace.expected)]
+    check(folders[name], dtype, requests, trace, results)
+
+
+# ---------------------------------------------------------------------------------------------- generation
+def plain_greedy(folder, dtype, prompt, steps):
+    history, out = list(prompt), []
+    for _ in range(steps):
+        token = int(np.argmax(BH.plain_logits(folder, dtype, history)[-1]))
+        history.append(token)
+        out.append(token)
+    return out
+
+
+def test_greedy_generation_through_the_entry_point(folders):
+    """Prompts of 1 to 70 tokens in portions of 16, 20 greedy tokens each, float32: every token is the plain side's."""
+    from sprout_lm_amd.engine import Engine
+    for name in ("general", "odd"):
+        engine = Engine.from_folder(folders[name], "float32", block_size=BH.PAGE[name], num_blocks=64, max_sequences=4,
+                                    max_batch_tokens=48, prefill_chunk_size=16, record_trace=True)
+        vocab = BH.CONFIGS[name]["vocab"]
+        prompts = [BH.random_tokens(vocab, n, 40 + i) for i, n in enumerate((1, 9, 40, 70))]
+        outputs = engine.generate(prompts, max_new_tokens=20, ignore_eos=True)
+        for prompt, got in zip(prompts, outputs):
+            assert got == plain_greedy(folders[name], "float32", prompt, 20), f"{name}, prompt of {len(prompt)}"
+        engine.cache.clear_prefixes()      # pages of finished prompts stay for later requests with the same beginning
+        assert all(free == g.pool.num_pages for free, g in zip(engine.cache.free_pages(), engine.cache.groups))
+
+
+def test_shared_prefix_pages_give_the_same_tokens(folders):
+    """A request whose prompt begins like an earlier one's takes over that one's pages (keys and the blended values are
+    functions of the tokens before them alone; blocks of the mask shorter than a prompt give some pages back first) and
+    generates what it generates alone."""
+    from sprout_lm_amd.engine import Engine
+    name, dtype = "general", "float32"
+    vocab = BH.CONFIGS[name]["vocab"]
+    common = BH.random_tokens(vocab, 83, 5)
+    prompts = [common + BH.random_tokens(vocab, n, 6 + n) for n in (3, 11, 1)]
+    engine = Engine.from_folder(folders[name], dtype, block_size=8, num_blocks=96, max_sequences=4, max_batch_tokens=64,
+                                prefill_chunk_size=32, record_trace=True)
+    first = engine.generate([prompts[0]], max_new_tokens=8, ignore_eos=True)
+    later = engine.generate(prompts[1:], max_new_tokens=8, ignore_eos=True)
+    for prompt, got in zip(prompts, first + later):
+        assert got == plain_greedy(folders[name], dtype, prompt, 8)
+    assert engine.scheduler.stats["prefix_hit_tokens"] >= 2 * 80, "the later requests found no pages of the first"
+
+
+def test_scheduling_never_changes_generation(folders):
+    """Too few pages (preemption, then the prompt and what was generated computed again) and a late arrival give what
+    each request generates alone."""
+    from sprout_lm_amd.engine import Engine
+    name, dtype = "general", "float32"
+    vocab = BH.CONFIGS[name]["vocab"]
+    prompts = {"A": BH.random_tokens(vocab, 33, 78), "B": BH.random_tokens(vocab, 29, 79),
+               "C": BH.random_tokens(vocab, 40, 80), "D": BH.random_tokens(vocab, 3, 81)}
+    want = {k: plain_greedy(folders[name], dtype, p, 14) for k, p in prompts.items()}
+    for num_blocks, expect_preemption in ((64, False), (12, True)):
+        engine = Engine.from_folder(folders[name], dtype, block_size=8, num_blocks=num_blocks, max_sequences=4,
+                                    max_batch_tokens=24, prefill_chunk_size=16, record_trace=True)
+        engine.add("A", prompts["A"], 14, ignore_eos=True)
+        engine.step(); engine.step(); engine.step()
+        for k in "BCD":
+            engine.add(k, prompts[k], 14, ignore_eos=True)
+        ticks = 0
+        while engine.pending:
+            ticks += 1
+            assert ticks < 2000
+            engine.step()
+        for k in prompts:
+            assert engine.result(k)["output"] == want[k], f"request {k} with {num_blocks} pages"
+        assert any(e["type"] == "preempted" for e in engine.trace) == expect_preemption
+
+
+def test_recorded_steps_equal_eager_steps(folders):
+    """Steps replayed from recorded graphs (decoded tokens with the sampler inside, portions of recurring shapes) give
+    the tokens of eagerly launched steps."""
+    from sprout_lm_amd.engine import Engine
+    name = "all_chosen"
+    vocab = BH.CONFIGS[name]["vocab"]
+    prompts = [BH.random_tokens(vocab, n, 60 + i) for i, n in enumerate((7, 21, 3, 40, 12))]
+
+    def run(use_graphs):
+        engine = Engine.from_folder(folders[name], "bfloat16", block_size=16, num_blocks=48, max_sequences=4,
+                                    max_batch_tokens=32, prefill_chunk_size=16)
+        engine.model.use_graphs = use_graphs
+        engine.add("r0", prompts[0], 30, ignore_eos=True)
+        engine.add("r1", prompts[1], 25, ignore_eos=True)
+        steps = 0
+        while engine.pending:
+            steps += 1
+            if steps == 6:
+                engine.add("r2", prompts[2], 20, temperature=0.8, seed=5, ignore_eos=True)
+            if steps == 15:
+                engine.add("r3", prompts[3], 10, ignore_eos=True)
+                engine.add("r4", prompts[4], 28, temperature=1.2, seed=9, ignore_eos=True)
+            engine.step()
+        replays = engine.model._graphs.replays if engine.model._graphs else 0
+        return [engine.result(f"r{i}")["output"] for i in range(5)], replays
+
+    eager, none = run(False)
+    graphed, replays = run(True)
+    assert none == 0 and replays > 40
+    assert graphed == eager
+
+
+def test_command_line_generates(folders):
+    done = subprocess.run([sys.executable, "-m", "sprout_lm_amd", "generate", folders["general"], "--prompt-ids",
+                           "3,1,4,1,5,9,2,6", "--dtype", "float32", "--ignore-eos"], cwd=ROOT,
+                          env=dict(os.environ, MAX_NEW_TOKENS="6"), capture_output=True, text=True, timeout=120)
+    assert done.returncode == 0, done.stderr
+    final = json.loads(done.stdout.strip().splitlines()[-1])
+    assert final["output"] == plain_greedy(folders["general"], "float32", [3, 1, 4, 1, 5, 9, 2, 6], 6)
