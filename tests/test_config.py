@@ -93,8 +93,13 @@ def test_sizes_that_no_kernel_takes_are_refused_when_the_parts_are_built():
         PartPlan("feed_forward", "gated_mlp", {"hidden": 8, "inner": 8, "activation": "gelu"}).make()
     with pytest.raises(ops.KernelError, match="rotation pairing 'interleaved'"):
         ops.kernels.variant_code(ops.ROTARY_PAIRINGS, "interleaved", "rotation pairing")
-    assert ops.ROTARY_PAIRINGS == {"halves": 0} and ops.GATE_ACTIVATIONS == {"silu": 0}
+    assert ops.ROTARY_PAIRINGS == {"halves": 0} and ops.GATE_ACTIVATIONS == {"silu": 0, "clamped_swish": 1}
+    with pytest.raises(ValueError, match="needs a positive limit"):
+        PartPlan("feed_forward", "gated_mlp", {"hidden": 8, "inner": 8, "activation": "clamped_swish"}).make()
     with pytest.raises(ConfigError, match="score stage 'soft_cap'"):
         PartPlan("mixer", "attention", {"hidden": 32, "heads": 2, "kv_heads": 1, "head_dim": 16, "scores": "soft_cap",
                                         "position": PartPlan("position", "none", {"head_dim": 16})}).make()
-    assert ops.SCORE_STAGES == {"scaled_dot": 0}
+    with pytest.raises(ConfigError, match="need a positive cap"):
+        PartPlan("mixer", "attention", {"hidden": 32, "heads": 2, "kv_heads": 1, "head_dim": 16, "scores": "capped",
+                                        "position": PartPlan("position", "none", {"head_dim": 16})}).make()
+    assert ops.SCORE_STAGES == {"scaled_dot": 0, "capped": 1}
