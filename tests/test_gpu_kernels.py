@@ -558,10 +558,12 @@ def test_variants_without_a_kernel_are_refused_by_the_library_itself():
     assert lib.sp_rope_cache(*args, 1) != 0 and b"pairing 1" in lib.sp_last_error()
     gu = torch.zeros(2, 32, device=DEV)
     out = torch.zeros(2, 16, device=DEV)
-    assert lib.sp_silu_mul(stream, 0, gu.data_ptr(), out.data_ptr(), 2, 16, 0) == 0
-    assert lib.sp_silu_mul(stream, 0, gu.data_ptr(), out.data_ptr(), 2, 16, 3) != 0 and b"activation 3" in lib.sp_last_error()
+    assert lib.sp_silu_mul(stream, 0, gu.data_ptr(), out.data_ptr(), 2, 16, 0, 0.0, None, 0) == 0
+    assert lib.sp_silu_mul(stream, 0, gu.data_ptr(), out.data_ptr(), 2, 16, 1, 1.5, None, 0) == 0
+    assert lib.sp_silu_mul(stream, 0, gu.data_ptr(), out.data_ptr(), 2, 16, 3, 0.0, None, 0) != 0 and b"activation 3" in lib.sp_last_error()
     assert lib.sp_fused_supported(ops.FUSED_ROPE, 8, 1152, 896, 64, 64, 0, 0) == 1
     assert lib.sp_fused_supported(ops.FUSED_ROPE, 8, 1152, 896, 64, 64, 0, 1) == 0
+    assert lib.sp_fused_supported(ops.FUSED_SILU, 8, 9728, 896, 0, 0, 0, 1) == 1
     assert lib.sp_fused_supported(ops.FUSED_SILU, 8, 9728, 896, 0, 0, 0, 2) == 0
     assert not ops.fused_supported(ops.FUSED_SILU, 8, 9728, 896, variant="gelu")
     with pytest.raises(ops.KernelError, match="activation 'relu'"):
@@ -574,6 +576,8 @@ def test_variants_without_a_kernel_are_refused_by_the_library_itself():
     assert ops.attention(q, 32, kp, vp, tables, batch, torch.zeros_like(q), 2, 1, 16, None, 0.25) is False
     with pytest.raises(ops.KernelError, match="score stage 'soft_cap'"):
         ops.attention(q, 32, kp, vp, tables, batch, torch.zeros_like(q), 2, 1, 16, None, 0.25, scores="soft_cap")
+    with pytest.raises(ops.KernelError, match="positive cap"):
+        ops.attention(q, 32, kp, vp, tables, batch, torch.zeros_like(q), 2, 1, 16, None, 0.25, scores="capped")
     torch.cuda.synchronize()
 
 
