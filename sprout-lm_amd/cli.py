@@ -2,7 +2,7 @@
 
     python -m sprout_lm_amd demo [--json] [--pressure]
     python -m sprout_lm_amd generate MODEL_DIR --prompt-ids 1,2,3 [--max-new-tokens N] ...
-    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b|megozen-s|... | --config FILE  --out DIR [--seed N]
+    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b|megozen-s|bogilix-s|... | --config FILE  --out DIR [--seed N]
 
 `demo` is the counterpart of the reference's src/demo.ts, with the reference's two options: a few requests on a
 tiny random model, told round by round (--json: the same as one JSON document; --pressure: a pool so small that
@@ -78,6 +78,40 @@ PRESETS.update({
     # large: 8 layers of width 4,096, 32 heads over one latent
     "megozen-l": _megozen_preset(4096, 8, 32, 64, 32, 64, 96, 64, 6, 1024, 2048, None, 32768),
     "megozen-l-dense": _dense_twin(4096, 8, 32, 4, 8192, 32768),
+})
+
+
+def _bogilix_preset(width: int, layers: int, heads: int, kv_heads: int, dim: int, normed_dim: int, chunk: int, experts: int,
+                    identity: int, top: int, ff: int, shared_ff: int, dense_ff: int, vocab: int) -> dict:
+    """A Bogilix configuration: three layers with normed queries and keys (heads of `normed_dim`, capped scores) to one
+    with rotated ones (heads of `dim`), values of `dim`, blocks of `chunk` positions (twice that in the rotated layers);
+    the first layer's feed-forward dense, the others routed (four groups of which two stay open)."""
+    def mixer(kind):
+        m = {"heads": heads, "kv_heads": kv_heads, "vdim": dim, "v_mix": True}
+        if kind == "attention":
+            m.update({"dim": dim, "scale": dim ** -0.5, "mask": {"size": 2 * chunk}, "rot": {"base": 500000.0, "dims": dim}})
+        else:
+            m.update({"dim": normed_dim, "scale": normed_dim ** -0.5, "mask": {"size": chunk}, "softcap": 50.0})
+        return m
+    moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": shared_ff, "limit": 7.0},
+           "router": {"experts": experts, "identity": identity, "top": top, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    entries = []
+    for i in range(layers):
+        kind = "attention" if i % 4 == 3 else "attention_2"
+        entries.append({"type": kind, "mixer": mixer(kind), "mlp": {"kind": "dense", "ff": dense_ff} if i == 0 else moe})
+    return {"architecture": "Bogilix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "layers": entries}
+
+
+PRESETS.update({
+    # small: 8 layers of width 1,024, 16 heads of 64 over 2 key/value heads, blocks of 1,024 and 2,048 positions
+    "bogilix-s": _bogilix_preset(1024, 8, 16, 2, 64, 48, 1024, 14, 2, 2, 512, 1024, 2048, 32768),
+    "bogilix-s-dense": _dense_twin(1024, 8, 16, 2, 2048, 32768),
+    # medium: 12 layers of width 2,048, 16 heads of 128 (normed layers: keys of 96 beside values of 128)
+    "bogilix-m": _bogilix_preset(2048, 12, 16, 2, 128, 96, 1024, 30, 2, 4, 704, 1408, 4224, 32768),
+    "bogilix-m-dense": _dense_twin(2048, 12, 16, 2, 4224, 32768),
+    # large: 8 layers of width 4,096, 32 heads of 128 over 4 key/value heads
+    "bogilix-l": _bogilix_preset(4096, 8, 32, 4, 128, 128, 2048, 62, 2, 6, 1024, 2048, 8192, 32768),
+    "bogilix-l-dense": _dense_twin(4096, 8, 32, 4, 8192, 32768),
 })
 
 

@@ -268,23 +268,17 @@ __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restr
   const int t = blockIdx.x;
   const int32_t* rows = row_of_pair + size_t(t) * top;
   const float* wt = weights + size_t(t) * top;
-  if (ids) {
-    const int32_t* id = ids + size_t(t) * top;
-    const TX* own = x + size_t(t) * H;
-    for (int i = blockIdx.y * 1024 + threadIdx.x; i < min(H, (int(blockIdx.y) + 1) * 1024); i += 256) {
-      float sum = 0.f;
-      for (int k = 0; k < top; ++k) sum = fmaf(wt[k], id[k] >= real ? to_float(own[i]) : y[size_t(rows[k]) * H + i], sum);
-      residual[size_t(t) * H + i] += sum;
-    }
-    return;
-  }
+  const int32_t* id = ids ? ids + size_t(t) * top : nullptr;
+  const TX* own = ids ? x + size_t(t) * H : nullptr;
   if ((H & 3) == 0) {
     const int i = 4 * (blockIdx.y * 256 + threadIdx.x);
     if (i >= H) return;
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int k = 0; k < top; ++k) {
       const float w = wt[k];
-      const float4 v = *reinterpret_cast<const float4*>(y + size_t(rows[k]) * H + i);
+      float4 v;
+      if (id && id[k] >= real) v = make_float4(to_float(own[i]), to_float(own[i + 1]), to_float(own[i + 2]), to_float(own[i + 3]));
+      else v = *reinterpret_cast<const float4*>(y + size_t(rows[k]) * H + i);
       sum.x = fmaf(w, v.x, sum.x); sum.y = fmaf(w, v.y, sum.y); sum.z = fmaf(w, v.z, sum.z); sum.w = fmaf(w, v.w, sum.w);
     }
     float4* r = reinterpret_cast<float4*>(residual + size_t(t) * H + i);
@@ -294,7 +288,7 @@ __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restr
   }
   for (int i = blockIdx.y * 1024 + threadIdx.x; i < min(H, (int(blockIdx.y) + 1) * 1024); i += 256) {
     float sum = 0.f;
-    for (int k = 0; k < top; ++k) sum = fmaf(wt[k], y[size_t(rows[k]) * H + i], sum);
+    for (int k = 0; k < top; ++k) sum = fmaf(wt[k], id && id[k] >= real ? to_float(own[i]) : y[size_t(rows[k]) * H + i], sum);
     residual[size_t(t) * H + i] += sum;
   }
 }

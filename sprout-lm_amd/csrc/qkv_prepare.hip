@@ -28,79 +28,98 @@ struct PrepareArgs {
   void* q_out;                 // [T, nq * width]
 };
 
-// One block a token.
+// Sum of the squares of n numbers over the whole block, as the scale of an RMS norm; every thread gets it.
 template <typename T>
-__global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepareArgs a) {
-  __shared__ float scratch[16];
-  const int t = blockIdx.x;
+__device__ __forceinline__ float row_scale(const T* __restrict__ x, int n, float eps, float* scratch) {
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = to_float(x[i]); sq = fmaf(v, v, sq); }
+  return 1.0f / sqrtf(block_sum(sq, scratch) / float(n) + eps);
+}
+
+// One head of one token (query heads, then key heads, then value heads), by `count` threads of which this is `lane`.
+template <typename T>
+__device__ __forceinline__ void prepare_head(const PrepareArgs& a, int t, int head, float q_scale, float k_scale, int slot,
+                                             int lane, int count) {
   const T* row = (const T*)a.proj + size_t(t) * a.stride;
   const int nq = a.nq, nkv = a.nkv, D = a.dim, V = a.vdim, W = a.width;
-  const T* qrow = row;
-  const T* krow = row + size_t(nq) * D;
-  const T* vrow = krow + size_t(nkv) * D;
-  float q_scale = 1.f, k_scale = 1.f;
-  if (a.q_norm) {
-    float sq = 0.f;
-    for (int i = threadIdx.x; i < nq * D; i += blockDim.x) { const float x = to_float(qrow[i]); sq = fmaf(x, x, sq); }
-    q_scale = 1.0f / sqrtf(block_sum(sq, scratch) / float(nq * D) + a.eps);
-    sq = 0.f;
-    for (int i = threadIdx.x; i < nkv * D; i += blockDim.x) { const float x = to_float(krow[i]); sq = fmaf(x, x, sq); }
-    k_scale = 1.0f / sqrtf(block_sum(sq, scratch) / float(nkv * D) + a.eps);
-  }
-  const int slot = a.slot_mapping ? a.slot_mapping[t] : -1;
   const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
+  if (head >= nq + nkv) {
+    // values: blended with the first flagged layer's, or kept for the later layers; written dimension-major
+    const int g = head - nq - nkv;
+    const T* vrow = row + size_t(nq + nkv) * D + size_t(g) * V;
+    const float lam = a.blend ? to_float(*(const T*)a.blend) : 0.f;
+    T* first = a.first ? (T*)a.first + size_t(t) * nkv * V + size_t(g) * V : nullptr;
+    for (int d = lane; d < W; d += count) {
+      float v = 0.f;
+      if (d < V) {
+        v = to_float(vrow[d]);
+        if (a.blend) v = to_float(from_float<T>((1.0f - lam) * v + lam * to_float(first[d])));
+        else if (a.keep_first) first[d] = from_float<T>(v);
+      }
+      if (slot >= 0) ((T*)a.v_pool)[((size_t(page) * nkv + g) * W + d) * a.page_size + off] = from_float<T>(v);
+    }
+    return;
+  }
+  const bool is_q = head < nq;
+  if (!is_q && slot < 0) return;        // a key that nobody keeps
+  const T* src = row + size_t(head) * D;                  // key heads follow the query heads in the row
+  const T* nw = is_q ? (const T*)a.q_norm : (const T*)a.k_norm;
+  if (nw) nw += size_t(is_q ? head : head - nq) * D;
+  const float scale = is_q ? q_scale : k_scale;
+  T* dst = is_q ? (T*)a.q_out + (size_t(t) * nq + head) * W
+                : (T*)a.k_pool + ((size_t(page) * nkv + (head - nq)) * a.page_size + off) * W;
   const int half = a.rotary_dim / 2;
-  const int pos = a.positions ? a.positions[t] : 0;
-
-  // queries and keys: head by head, number by number of the padded head; a thread that owns the first of a turning
-  // pair also writes its partner
-  const int heads = nq + nkv;
-  for (int i = threadIdx.x; i < heads * W; i += blockDim.x) {
-    const int head = i / W, d = i % W;
-    const bool is_q = head < nq;
-    T* dst = nullptr;
-    if (is_q) dst = (T*)a.q_out + (size_t(t) * nq + head) * W;
-    else if (slot >= 0) dst = (T*)a.k_pool + ((size_t(page) * nkv + (head - nq)) * a.page_size + off) * W;
-    if (!dst) continue;
+  auto normed = [&](int e) {
+    float x = to_float(src[e]);
+    if (nw) x = to_float(from_float<T>((x * scale) * to_float(nw[e])));   // the storage type's rounding, as a norm kernel would leave it
+    return x;
+  };
+  for (int d = lane; d < W; d += count) {
     if (d >= D) { dst[d] = from_float<T>(0.f); continue; }
-    if (d >= half && d < 2 * half) continue;          // written by the owner of its pair
-    const T* src = is_q ? qrow + size_t(head) * D : krow + size_t(head - nq) * D;
-    const T* nw = is_q ? (const T*)a.q_norm : (const T*)a.k_norm;
-    const float scale = is_q ? q_scale : k_scale;
-    const int col = (is_q ? head : head - nq) * D;
-    auto normed = [&](int e) {
-      float x = to_float(src[e]);
-      if (nw) x = to_float(from_float<T>((x * scale) * to_float(nw[col + e])));   // the storage type's rounding, as a norm kernel would leave it
-      return x;
-    };
     if (d >= 2 * half) { dst[d] = from_float<T>(normed(d)); continue; }
+    if (d >= half) continue;          // written by the owner of its pair
     float sn, cs;
     if (a.inv_freq_tail) {
       double sn64, cs64;
-      sincos(double(pos) * (double(a.inv_freq[d]) + double(a.inv_freq_tail[d])), &sn64, &cs64);
+      sincos(double(a.positions[t]) * (double(a.inv_freq[d]) + double(a.inv_freq_tail[d])), &sn64, &cs64);
       sn = float(sn64);
       cs = float(cs64);
     } else {
-      sincosf(float(pos) * a.inv_freq[d], &sn, &cs);
+      sincosf(float(a.positions[t]) * a.inv_freq[d], &sn, &cs);
     }
     const float x = normed(d), y = normed(d + half);
     dst[d] = from_float<T>(x * cs - y * sn);
     dst[d + half] = from_float<T>(y * cs + x * sn);
   }
+}
 
-  // values: blended with the first flagged layer's, kept for the later layers, written dimension-major
-  const float lam = a.blend ? to_float(*(const T*)a.blend) : 0.f;
-  T* first = a.first ? (T*)a.first + size_t(t) * nkv * V : nullptr;
-  for (int i = threadIdx.x; i < nkv * W; i += blockDim.x) {
-    const int g = i / W, d = i % W;
-    float v = 0.f;
-    if (d < V) {
-      v = to_float(vrow[g * V + d]);
-      if (a.blend) v = to_float(from_float<T>((1.0f - lam) * v + lam * to_float(first[g * V + d])));
-      else if (a.keep_first) first[g * V + d] = from_float<T>(v);
-    }
-    if (slot >= 0) ((T*)a.v_pool)[((size_t(page) * nkv + g) * W + d) * a.page_size + off] = from_float<T>(v);
+// PER_HEAD: one block per (token, head), for the few tokens of a decode step: the work still spreads over the chip and
+// every block waits for memory once; a block of a normed head sums the squares of its whole row by itself (a few
+// kilobytes that the other heads' blocks read at the same time).  Otherwise one block a token: the row's two sums
+// are taken once, and the block's waves take the heads in turn.
+template <typename T, bool PER_HEAD>
+__global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepareArgs a) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const T* row = (const T*)a.proj + size_t(t) * a.stride;
+  const int slot = a.slot_mapping ? a.slot_mapping[t] : -1;
+  const int heads = a.nq + 2 * a.nkv;
+  if (PER_HEAD) {
+    const int head = blockIdx.y;
+    float scale = 1.f;
+    if (a.q_norm && head < a.nq + a.nkv && (head < a.nq || slot >= 0))
+      scale = head < a.nq ? row_scale(row, a.nq * a.dim, a.eps, scratch)
+                          : row_scale(row + size_t(a.nq) * a.dim, a.nkv * a.dim, a.eps, scratch);
+    prepare_head<T>(a, t, head, scale, scale, slot, threadIdx.x, blockDim.x);
+    return;
   }
+  float q_scale = 1.f, k_scale = 1.f;
+  if (a.q_norm) {
+    q_scale = row_scale(row, a.nq * a.dim, a.eps, scratch);
+    k_scale = row_scale(row + size_t(a.nq) * a.dim, a.nkv * a.dim, a.eps, scratch);
+  }
+  const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  for (int head = wave; head < heads; head += waves) prepare_head<T>(a, t, head, q_scale, k_scale, slot, threadIdx.x & 63, 64);
 }
 
 }  // namespace sprout
@@ -125,8 +144,16 @@ extern "C" int sp_qkv_prepare(void* stream, int dtype, const void* proj, long lo
   PrepareArgs a = {proj, stride, nq, nkv, dim, vdim, width, q_norm, k_norm, eps, positions, inv_freq, inv_freq_tail, rotary_dim,
                    blend, first, keep_first, slot_mapping, k_pool, v_pool, page_size, q_out};
   hipStream_t s = (hipStream_t)stream;
-  if (dtype == kF32) qkv_prepare_kernel<float><<<T, 256, 0, s>>>(a);
-  else if (dtype == kBF16) qkv_prepare_kernel<bf16_t><<<T, 256, 0, s>>>(a);
-  else SP_REQUIRE(false, "sp_qkv_prepare: unsupported dtype %d", dtype);
+  SP_REQUIRE(nq + 2 * nkv <= 65535, "sp_qkv_prepare: %d heads are more than a launch's second dimension holds", nq + 2 * nkv);
+  SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_qkv_prepare: unsupported dtype %d", dtype);
+  if (T * (nq + 2 * nkv) <= 2048) {      // few tokens: a block per head
+    const dim3 grid(T, nq + 2 * nkv);
+    const int threads = width <= 64 ? 64 : 128;
+    if (dtype == kF32) qkv_prepare_kernel<float, true><<<grid, threads, 0, s>>>(a);
+    else qkv_prepare_kernel<bf16_t, true><<<grid, threads, 0, s>>>(a);
+  } else {
+    if (dtype == kF32) qkv_prepare_kernel<float, false><<<T, 256, 0, s>>>(a);
+    else qkv_prepare_kernel<bf16_t, false><<<T, 256, 0, s>>>(a);
+  }
   return check_launch("sp_qkv_prepare");
 }
