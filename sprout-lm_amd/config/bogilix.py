@@ -104,10 +104,13 @@ class FeedForwardSizes:
         if kind != "moe":
             raise ConfigError(f"{_WHAT}{where}kind must be 'dense' or 'moe', got {kind!r}.")
         expert, router = _section(raw, "expert", where), _section(raw, "router", where)
-        groups = _section(router, "groups", where + "router.")
-        experts, identity = _count(router, "experts", where + "router."), _count(router, "identity", where + "router.", 0)
+        # a router without identity experts or without groups may leave those keys out: no experts of that kind, one group
+        groups = _section(router, "groups", where + "router.", optional=True)
+        experts = _count(router, "experts", where + "router.")
+        identity = _count(router, "identity", where + "router.", 0) if router.get("identity") is not None else 0
         top = _count(router, "top", where + "router.")
-        count, keep = _count(groups, "count", where + "router.groups."), _count(groups, "keep", where + "router.groups.")
+        count, keep = (1, 1) if groups is None else (_count(groups, "count", where + "router.groups."),
+                                                     _count(groups, "keep", where + "router.groups."))
         outputs = experts + identity
         if outputs % count or keep > count or top > keep * (outputs // count):
             raise ConfigError(f"{_WHAT}{where}router: {outputs} outputs do not form {count} equal groups of which {keep} "

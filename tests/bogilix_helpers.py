@@ -72,9 +72,16 @@ DENSE = model(64, 150, [
     layer(normed(2, 1, 48, 80, 0.1, 9, 50.0)),
 ])
 
-CONFIGS = {"odd": ODD, "general": GENERAL, "all_chosen": ALL_CHOSEN, "dense": DENSE}
-PAGE = {"odd": 16, "general": 16, "all_chosen": 8, "dense": 4}
-SEED = {"odd": 14, "general": 15, "all_chosen": 16, "dense": 17}
+# sizes in no whole eights again, and nothing discrete: dense feed-forwards and routers that choose everything (bfloat16)
+ODD_SAFE = model(100, 77, [
+    layer(rotary(3, 3, 20, 6, 0.4, 7, 8, base=300.0), moe(3, 1, 4, 2, 2, 1.5, 28, 0.8, shared=(20, 1.2))),
+    layer(normed(6, 2, 12, 10, 0.3, 5, 7.0, v_mix=True), dense(28)),
+    layer(normed(5, 1, 6, 20, 0.9, 37, 2.5, v_mix=True)),
+], eps=1e-3)
+
+CONFIGS = {"odd": ODD, "odd_safe": ODD_SAFE, "general": GENERAL, "all_chosen": ALL_CHOSEN, "dense": DENSE}
+PAGE = {"odd": 16, "odd_safe": 16, "general": 16, "all_chosen": 8, "dense": 4}
+SEED = {"odd": 14, "odd_safe": 18, "general": 15, "all_chosen": 16, "dense": 17}
 
 
 def random_weights(cfg: dict, seed: int) -> dict:

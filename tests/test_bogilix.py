@@ -47,6 +47,14 @@ def test_configuration_refusals(path, value):
         S.config_from_dict(broken(path, value))
 
 
+def test_router_keys_that_may_be_left_out():
+    raw = copy.deepcopy(BH.CONFIGS["general"])
+    router = raw["layers"][1]["mlp"]["router"]
+    del router["identity"], router["groups"]
+    mlp = S.config_from_dict(raw).layers[1].mlp
+    assert (mlp.identity, mlp.groups, mlp.keep) == (0, 1, 1)
+
+
 def test_plan_names_every_tensor_and_cache_slot():
     from sprout_lm_amd.cache.spec import PagedKVSpec
     from sprout_lm_amd.parts.sink_attention import padded_width

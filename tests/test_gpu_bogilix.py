@@ -189,6 +189,7 @@ ATT_SHAPES = [  # nq, nkv, dim, vdim, chunk, cap, page
     (32, 1, 16, 32, 16, 4.0, 16),     # more heads than a block of the one-query kernel holds
     (3, 3, 20, 6, 5, None, 4),        # a width only the general kernel takes
     (6, 2, 12, 10, 300, 7.0, 16),     # blocks longer than a chunk of the one-query kernels
+    (2, 1, 136, 150, 20, 3.0, 8),     # heads wider than the bfloat16 matrix-core kernels take
 ]
 
 
@@ -452,9 +453,9 @@ def check(folder, dtype, requests, trace, results):
     return worst
 
 
-LENGTHS = {"odd": [1, 2, 21, 70, 45, 97], "general": [1, 9, 40, 97, 150, 33, 2, 75], "all_chosen": [9, 40, 97, 33, 130],
+LENGTHS = {"odd": [1, 2, 21, 70, 45, 97], "odd_safe": [1, 2, 21, 70, 45, 97], "general": [1, 9, 40, 97, 150, 33, 2, 75], "all_chosen": [9, 40, 97, 33, 130],
            "dense": [2, 70, 97, 33, 64, 120]}
-CASES = [(n, "float32") for n in BH.CONFIGS] + [("all_chosen", "bfloat16"), ("dense", "bfloat16")]
+CASES = [(n, "float32") for n in BH.CONFIGS] + [("all_chosen", "bfloat16"), ("dense", "bfloat16"), ("odd_safe", "bfloat16")]
 
 
 @pytest.mark.parametrize("name,dtype", CASES)
