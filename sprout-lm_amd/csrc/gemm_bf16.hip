@@ -160,7 +160,8 @@ int gemm_decode_plain(hipStream_t s, const void* x, const void* w, int bias_dtyp
 bool gemm_pipe_takes(int T, int N, int K);
 int gemm_bf16_pipe(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, void* out,
                    int T, int N, int K);
-int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit);
+int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit,
+                        const float* row_gate, long long row_gate_stride);
 
 // mode 0 stores bfloat16 here; a float32 store of mode 0 is passed in as mode 2 by the caller.
 int gemm_bf16(hipStream_t s, const void* a, const void* w, int bias_dtype, const void* bias, int mode, int out_dtype,
@@ -365,9 +366,10 @@ static int tiled_shape(hipStream_t s, const void* x, const void* w, const void* 
 
 // out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T): the pipelined kernel where it takes the shape, else (T > 64)
 // this file's kernel with 128-token tiles, 64 gate + 64 up rows per block.
-int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit) {
-  if (gemm_pipe_takes(T, 2 * I, K)) return gemm_bf16_pipe_silu(s, x, w, out, T, I, K, act, limit);
-  SP_REQUIRE(act == kActSilu, "sp_gate_up_silu: the tiles for K=%d have the SiLU epilogue alone", K);
+int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit,
+                         const float* row_gate, long long row_gate_stride) {
+  if (gemm_pipe_takes(T, 2 * I, K)) return gemm_bf16_pipe_silu(s, x, w, out, T, I, K, act, limit, row_gate, row_gate_stride);
+  SP_REQUIRE(act == kActSilu && !row_gate, "sp_gate_up_silu: the tiles for K=%d have the SiLU epilogue alone", K);
   dim3 grid((I + 63) / 64, (T + 127) / 128, 1);
   return launch_tiled_mode<2, 2, 64, kSilu, float>(s, grid, (const uint16_t*)x, (const uint16_t*)w, nullptr, out, T, I, K,
                                                     (K + 63) / 64 * 64);

@@ -20,6 +20,8 @@ struct RopeArgs {
   // the gated epilogue (kSilu) reads only these: which activation (GateAct of common.h; 0 = SiLU) and its limit
   int act;
   float limit;
+  const float* row_gate;         // may be null: a token's row is also multiplied by sigmoid(row_gate[t * row_gate_stride])
+  long long row_gate_stride;
 };
 
 // Orders a wave's LDS writes before its own later reads of what other lanes wrote (and the reverse).
@@ -116,6 +118,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[WM][WN], float* tu
     for (int i = 0; i < WM; ++i) {
       const int t = t0 + (wm * WM + i) * 32 + li;
       if (t >= T) continue;
+      const float row = rope.row_gate ? 1.0f / (1.0f + expf(-rope.row_gate[size_t(t) * rope.row_gate_stride])) : 1.0f;
 #pragma unroll
       for (int m = 0; m < WN / 2; ++m) {
 #pragma unroll
@@ -128,6 +131,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[WM][WN], float* tu
             const float g = to_float(bf16_t{f32_to_bf16_bits(acc[i][2 * m][4 * rg + r])});
             const float u = to_float(bf16_t{f32_to_bf16_bits(acc[i][(2 * m + 1) % WN][4 * rg + r])});
             v[r] = rope.act == kActSilu ? g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u : gated_value(g, u, rope.act, rope.limit);
+            if (rope.row_gate) v[r] *= row;
           }
           uint16_t* dst = reinterpret_cast<uint16_t*>(out) + size_t(t) * N + n;
           if (n + 4 <= N && (N & 3) == 0) *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));

@@ -96,6 +96,8 @@ struct SkinnyExtra {
   // kSilu: which gated activation (GateAct of common.h) and its limit
   int act;
   float limit;
+  const float* row_gate;        // may be null: a token's row is also multiplied by sigmoid(row_gate[t * row_gate_stride])
+  long long row_gate_stride;
 };
 
 template <int RT, int MODE, typename TB, bool NORM, int WAVES = 4>   // MODE: kStoreF32, kAccumulate, kSilu or kRope
@@ -269,7 +271,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_f32_skinny_kernel(const float
     const int t = threadIdx.x & 15, r = threadIdx.x >> 4, n = n0 + r;
     if (t >= T || n >= N) return;
     const float gate = joined(0, t + 16 * (r >> 2), r & 3), up = joined(0, t + 16 * (r >> 2) + 32, r & 3);
-    out[size_t(t) * N + n] = gated_value(gate, up, extra.act, extra.limit);
+    out[size_t(t) * N + n] = gated_value(gate, up, extra.act, extra.limit) *
+                             (extra.row_gate ? 1.0f / (1.0f + expf(-extra.row_gate[size_t(t) * extra.row_gate_stride])) : 1.0f);
     return;
   }
   if (MODE == kSilu) {
@@ -280,7 +283,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_f32_skinny_kernel(const float
       for (int e = 0; e < 4; ++e) {
         if (n + e >= N) break;
         const float gate = joined(2 * pair, l, e), up = joined(2 * pair + 1, l, e);
-        out[size_t(t) * N + n + e] = gated_value(gate, up, extra.act, extra.limit);
+        out[size_t(t) * N + n + e] = gated_value(gate, up, extra.act, extra.limit) *
+                                     (extra.row_gate ? 1.0f / (1.0f + expf(-extra.row_gate[size_t(t) * extra.row_gate_stride])) : 1.0f);
       }
     }
     return;
@@ -333,13 +337,15 @@ int skinny_shape(hipStream_t s, const float* x, const float* w, const void* bias
 // out[T, I] = silu(a . w[:I]^T) * (a . w[I:]^T) for up to 16 tokens, float32 throughout; a = x, or
 // rmsnorm(x) * norm_w where norm_w is given.
 int gemm_f32_gated(hipStream_t s, const float* x, const float* norm_w, float eps, const float* w, float* out, int T, int I, int K,
-                   int act, float limit) {
+                   int act, float limit, const float* row_gate, long long row_gate_stride) {
   const int pairs = (I + 15) / 16, steps = (K + 15) / 16;
   SkinnyExtra extra = {};
   extra.norm_w = norm_w;
   extra.eps = eps;
   extra.act = act;
   extra.limit = limit;
+  extra.row_gate = row_gate;
+  extra.row_gate_stride = row_gate_stride;
 #define SP_GATED(RT, NORM, BLOCKS) \
   gemm_f32_skinny_kernel<RT, kSilu, float, NORM><<<dim3(BLOCKS, 1), 256, 0, s>>>(x, w, nullptr, out, T, I, K, steps, extra)
   if (pairs >= 2048) {
@@ -399,12 +405,13 @@ extern "C" int sp_gate_up_silu_f32_takes(int T, int I, int K) { return T >= 1 &&
 // a decode step on the float32 path, in one kernel.  a = x (float32 [T, K]), or rmsnorm(x) * norm_w (float32 [K],
 // eps) where norm_w is given: the norm before the feed-forward folded in.
 extern "C" int sp_gate_up_silu_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, float* out,
-                                   int T, int I, int K, int activation, float limit) {
+                                   int T, int I, int K, int activation, float limit, const float* row_gate,
+                                   long long row_gate_stride) {
   SP_REQUIRE(activation >= 0 && activation < kGateActs, "sp_gate_up_silu_f32: no kernel for activation %d", activation);
   SP_REQUIRE(sp_gate_up_silu_f32_takes(T, I, K), "sp_gate_up_silu_f32: shape T=%d I=%d K=%d is not taken", T, I, K);
   SP_REQUIRE(x && w && out && (reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(norm_w)) % 16 == 0,
              "sp_gate_up_silu_f32: operands must be given and 16-byte aligned");
-  return gemm_f32_gated((hipStream_t)stream, x, norm_w, eps, w, out, T, I, K, activation, limit);
+  return gemm_f32_gated((hipStream_t)stream, x, norm_w, eps, w, out, T, I, K, activation, limit, row_gate, row_gate_stride);
 }
 
 // Whether sp_qkv_rope_cache_f32 takes the shape: up to 16 tokens, head sizes in 16s turned whole, pairing "halves".

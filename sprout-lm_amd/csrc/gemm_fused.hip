@@ -52,9 +52,12 @@ struct FusedArgs {
   uint16_t* v_pool;
   int nq, nkv, hd, page_size, rotary_dim;
   int page_shift;            // page_size == 1 << page_shift, or -1 where it is no power of two
-  // kEpiSilu: which gated activation (GateAct of common.h) and its limit
+  // kEpiSilu: which gated activation (GateAct of common.h) and its limit; row_gate (may be null): a token's row is
+  // also multiplied by sigmoid(row_gate[t * row_gate_stride]), float32
   int act;
   float limit;
+  const float* row_gate;
+  long long row_gate_stride;
 };
 
 // A bias value as it lies in memory (bfloat16 bits or float32 bits), and its value.  The two are kept apart
@@ -403,7 +406,9 @@ __global__ __launch_bounds__(256) void gemm_fused_kernel(FusedArgs a) {
         const float gv = summed(gate >> 4, gate & 15, tn), uv = summed(up >> 4, up & 15, tn);
         // the engine keeps gate and up as bfloat16 before the gated product; keep the same roundings
         const float g = to_float(bf16_t{f32_to_bf16_bits(gv)}), u = to_float(bf16_t{f32_to_bf16_bits(uv)});
-        reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(gated_value(g, u, a.act, a.limit));
+        float v = gated_value(g, u, a.act, a.limit);
+        if (a.row_gate) v *= 1.0f / (1.0f + expf(-a.row_gate[size_t(t) * a.row_gate_stride]));
+        reinterpret_cast<uint16_t*>(a.out)[size_t(t) * a.partner + n] = f32_to_bf16_bits(v);
       }
       continue;
     }
@@ -587,7 +592,8 @@ extern "C" int sp_gemm_decode(void* stream, const void* x, const float* residual
                               int N, int K);
 
 namespace sprout {
-int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit);
+int gemm_bf16_tiled_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit,
+                         const float* row_gate, long long row_gate_stride);
 bool gemm_pipe_takes(int T, int N, int K);
 bool gemm_pipe_rope_takes(int T, int N, int K, int hd);
 int gemm_bf16_pipe_rope(hipStream_t s, const void* x, const void* w, int bias_dtype, const void* bias, void* q_out,
@@ -692,7 +698,7 @@ extern "C" int sp_qkv_rope_cache(void* stream, const void* x, const float* resid
 // out[T, I] = silu(x . w_gate^T) * (x . w_up^T) with w = [gate rows; up rows] of [2 I, K].
 extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype,
                                const void* norm_w, float eps, const void* w, void* out, int T, int I, int K,
-                               int activation, float limit) {
+                               int activation, float limit, const float* row_gate, long long row_gate_stride) {
   SP_REQUIRE(activation >= 0 && activation < kGateActs, "sp_gate_up_silu: no kernel for activation %d", activation);
   SP_REQUIRE(sp_fused_supported(kEpiSilu, T, 2 * I, K, 0, 0, residual != nullptr, activation),
              "sp_gate_up_silu: shape T=%d I=%d K=%d is not taken", T, I, K);
@@ -705,12 +711,12 @@ extern "C" int sp_gate_up_silu(void* stream, const void* x, const float* residua
   const size_t weights = size_t(2) * I * K;
   const int fused_up_to = weights >= (size_t(200) << 20) ? 4 : weights >= (size_t(64) << 20) ? 8 : 16;
   if (T > 64 || (T > fused_up_to && !residual && gemm_pipe_takes(T, 2 * I, K)))
-    return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K, activation, limit);
+    return gemm_bf16_tiled_silu((hipStream_t)stream, x, w, out, T, I, K, activation, limit, row_gate, row_gate_stride);
   FusedArgs a = {};
   a.x = (const uint16_t*)x; a.residual = residual; a.norm_w = norm_w; a.norm_w_bf16 = norm_w_dtype == kBF16; a.eps = eps;
   a.w = (const uint16_t*)w; a.out = out;
   a.T = T; a.N = 2 * I; a.K = K; a.k_per_split = (K + 63) / 64 * 64; a.partner = I;
-  a.act = activation; a.limit = limit;
+  a.act = activation; a.limit = limit; a.row_gate = row_gate; a.row_gate_stride = row_gate_stride;
   a.rows_per_block = silu_rows_per_block(T, I, K, residual != nullptr);
   return fused_norm<kEpiSilu>((hipStream_t)stream, a, residual != nullptr, (I + a.rows_per_block - 1) / a.rows_per_block, 1);
 }

@@ -5,11 +5,14 @@
 namespace sprout {
 
 // out[T, I] = silu(x . w[:I]^T) * (x . w[I:]^T): a block's weight rows are half gate rows, half the matching up rows.
-int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit) {
+int gemm_bf16_pipe_silu(hipStream_t s, const void* x, const void* w, void* out, int T, int I, int K, int act, float limit,
+                        const float* row_gate, long long row_gate_stride) {
   const uint16_t *xp = (const uint16_t*)x, *wp = (const uint16_t*)w;
   RopeArgs epi = {};
   epi.act = act;
   epi.limit = limit;
+  epi.row_gate = row_gate;
+  epi.row_gate_stride = row_gate_stride;
   int shape, splits;
   pipe_choice(T, 2 * I, K, false, &shape, &splits, true);
   if (shape == 0) return launch_pipe_mode<4, 2, 2, 4, 2, kSilu, float>(s, 1, xp, wp, nullptr, out, T, I, K, K, epi);

@@ -54,9 +54,10 @@ int sp_qkv_rope_cache(void* stream, const void* x, const float* residual, int no
                       const float* cos_sin, int pairing);
 // out [T][half][2] = (cosine, sine) of positions[t] * inv_freq[d]: the same for every layer of a step.
 int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T);
-// out [T, I] = silu(x . w[:I]^T) * (x . w[I:]^T)
+// out [T, I] = act(x . w[:I]^T, x . w[I:]^T) (times sigmoid(row_gate[t * row_gate_stride]) where row_gate, float32, is given)
 int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
-                    const void* w, void* out, int T, int I, int K, int activation, float limit);
+                    const void* w, void* out, int T, int I, int K, int activation, float limit, const float* row_gate,
+                    long long row_gate_stride);
 
 // Rotates q and k heads of qkv[T, (nq + 2 nkv) * hd] in place (neox pairing, angle = position *
 // inv_freq[d]) and writes k and v of every token into the paged pools at slot_mapping[t]
@@ -136,7 +137,7 @@ int sp_qkv_prepare(void* stream, int dtype, const void* proj, long long stride, 
 //                          q_out [T, nq * hd], k and v into the paged pools at slot_mapping.  Head sizes in 16s.
 int sp_gate_up_silu_f32_takes(int T, int I, int K);
 int sp_gate_up_silu_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, float* out,
-                        int T, int I, int K, int activation, float limit);
+                        int T, int I, int K, int activation, float limit, const float* row_gate, long long row_gate_stride);
 int sp_qkv_rope_cache_f32_takes(int T, int K, int nq, int nkv, int hd, int rotary_dim, int pairing);
 int sp_qkv_rope_cache_f32(void* stream, const float* x, const float* norm_w, float eps, const float* w, int bias_dtype,
                           const void* bias, float* q_out, const int32_t* positions, const float* inv_freq,

@@ -716,19 +716,21 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tenso
 
 
 def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0,
-                 activation: str = "silu", limit: float = 0.0) -> None:
-    """out = act(a . w[:I]^T) * (a . w[I:]^T) for activations a as in `qkv_rope_cache`."""
+                 activation: str = "silu", limit: float = 0.0, row_gate=None, row_gate_column: int = 0) -> None:
+    """out = act(a . w[:I]^T, a . w[I:]^T) for activations a as in `qkv_rope_cache`, times sigmoid(row_gate[t, column])
+    where row_gate (float32 [T, columns]) is given."""
     _gpu(w, "gate/up weight"); _gpu(out, "gated output")
     N, K = w.shape
     xp, rp, nd, npt, T = _activations(x, residual, norm_weight, K, "gate_up_silu")
     if w.dtype != torch.bfloat16 or N % 2 or tuple(out.shape) != (T, N // 2) or out.dtype != torch.bfloat16:
         raise KernelError("gate_up_silu: weight [2 I, K] and output [T, I] bfloat16 expected")
     check(library().sp_gate_up_silu(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(), out.data_ptr(), T, N // 2, K,
-                                    variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit)))
+                                    variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit),
+                                    *_row_gate(row_gate, row_gate_column, T, "gate_up_silu")))
 
 
 def gate_up_silu_f32(w: torch.Tensor, x: torch.Tensor, out: torch.Tensor, activation: str = "silu", norm_weight=None,
-                     eps: float = 0.0, limit: float = 0.0) -> bool:
+                     eps: float = 0.0, limit: float = 0.0, row_gate=None, row_gate_column: int = 0) -> bool:
     """out = act(a . w[:I]^T) * (a . w[I:]^T), everything float32, for the few tokens of a decode step; a = x, or
     rmsnorm(x) * norm_weight computed inside the kernel where norm_weight is given (x is then the residual).  Returns
     False (and does nothing) where the kernel does not take the shape: the caller then multiplies and gates in turn."""
@@ -741,7 +743,8 @@ def gate_up_silu_f32(w: torch.Tensor, x: torch.Tensor, out: torch.Tensor, activa
         return False
     _gpu(w, "gate/up weight"); _gpu(x, "activations"); _gpu(out, "gated output")
     check(library().sp_gate_up_silu_f32(_stream(), x.data_ptr(), _ptr(norm_weight), float(eps), w.data_ptr(), out.data_ptr(),
-                                        T, I, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit)))
+                                        T, I, K, variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit),
+                                        *_row_gate(row_gate, row_gate_column, T, "gate_up_silu_f32")))
     return True
 
 
@@ -779,6 +782,16 @@ def qkv_rope_cache_f32(w: torch.Tensor, bias, x: torch.Tensor, q_out: torch.Tens
     return True
 
 
+def _row_gate(row_gate, column: int, T: int, what: str):
+    """(pointer, stride) of a float32 [>= T, columns] tensor's column, or (None, 0)."""
+    if row_gate is None:
+        return None, 0
+    _gpu(row_gate, "row gate")
+    if row_gate.dtype != torch.float32 or row_gate.dim() != 2 or row_gate.shape[0] < T or not 0 <= column < row_gate.shape[1]:
+        raise KernelError(f"{what}: the row gate must be float32 [>= T, columns]")
+    return row_gate.data_ptr() + 4 * column, row_gate.shape[1]
+
+
 def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu", limit: float = 0.0,
              row_gate: torch.Tensor | None = None, row_gate_column: int = 0) -> None:
     """out[t, i] = act(gu[t, i], gu[t, I + i]), times sigmoid(row_gate[t, row_gate_column]) where row_gate (float32
@@ -787,12 +800,7 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor, activation: str = "silu", limi
     T, I = out.shape
     if tuple(gu.shape) != (T, 2 * I) or gu.dtype != out.dtype:
         raise KernelError(f"silu_mul: shapes do not fit: gu {tuple(gu.shape)}, out {tuple(out.shape)}")
-    gate_ptr, gate_stride = None, 0
-    if row_gate is not None:
-        _gpu(row_gate, "row gate")
-        if row_gate.dtype != torch.float32 or row_gate.dim() != 2 or row_gate.shape[0] < T or not 0 <= row_gate_column < row_gate.shape[1]:
-            raise KernelError("silu_mul: the row gate must be float32 [>= T, columns]")
-        gate_ptr, gate_stride = row_gate.data_ptr() + 4 * row_gate_column, row_gate.shape[1]
+    gate_ptr, gate_stride = _row_gate(row_gate, row_gate_column, T, "silu_mul")
     check(library().sp_silu_mul(_stream(), _code(gu, "gate/up"), gu.data_ptr(), out.data_ptr(), T, I,
                                 variant_code(GATE_ACTIVATIONS, activation, "gate activation"), float(limit), gate_ptr, gate_stride))
 

@@ -76,10 +76,14 @@ class GatedMLP(FeedForward):
         the factor goes onto the gated product, of which the output is a linear function."""
         T = h.shape[0]
         act = ctx.buffer("gated", (T, self.inner), ctx.act_dtype)
-        if row_gate is None and ctx.act_dtype == torch.bfloat16 and self._fused(T, False):
-            ops.gate_up_silu(self.w_gate_up, act, x=h, activation=self.activation, limit=self.limit)
-        elif row_gate is None and ctx.act_dtype == torch.float32 and ops.gate_up_silu_f32(
-                self.w_gate_up, h, act, activation=self.activation, limit=self.limit):
+        # (the older tiles, for a K in no whole steps of 64, have no epilogue for a row gate or another activation)
+        plain = row_gate is None and self.activation == "silu"
+        if ctx.act_dtype == torch.bfloat16 and self._fused(T, False) and (plain or T <= 64 or self.hidden % 64 == 0):
+            ops.gate_up_silu(self.w_gate_up, act, x=h, activation=self.activation, limit=self.limit, row_gate=row_gate,
+                             row_gate_column=row_gate_column)
+        elif ctx.act_dtype == torch.float32 and ops.gate_up_silu_f32(
+                self.w_gate_up, h, act, activation=self.activation, limit=self.limit, row_gate=row_gate,
+                row_gate_column=row_gate_column):
             pass
         else:
             gu = ctx.buffer("gate_up", (T, 2 * self.inner), ctx.act_dtype)

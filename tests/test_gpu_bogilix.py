@@ -306,6 +306,9 @@ def test_clamped_gate_and_row_gate(dtype, T, I, K):
     residual = torch.zeros(T, K, dtype=torch.float32, device=DEV)
     part.forward(ctx, dev(x, dtype), residual)
     close(residual.cpu().numpy(), B.linear(store(want), down), dtype, "the part", f32=2e-5, bf16=2e-2)
+    residual.zero_()
+    part.forward(ctx, dev(x, dtype), residual, row_gate=dev(gate), row_gate_column=1)      # the gate folded into the product
+    close(residual.cpu().numpy(), B.linear(store(want * B.sigmoid(gate[:, 1:2])), down), dtype, "the part with a row gate", f32=2e-5, bf16=2e-2)
 
 
 def test_scored_routing_choice_ties_groups_and_identity():
