@@ -91,7 +91,7 @@ def _bogilix_preset(width: int, layers: int, heads: int, kv_heads: int, dim: int
         if kind == "attention":
             m.update({"dim": dim, "scale": dim ** -0.5, "mask": {"size": 2 * chunk}, "rot": {"base": 500000.0, "dims": dim}})
         else:
-            m.update({"dim": normed_dim, "scale": normed_dim ** -0.5, "mask": {"size": chunk}, "softcap": 50.0})
+            m.update({"dim": normed_dim, "scale": normed_dim ** -0.5, "mask": {"size": chunk}, "softcap": 30.0})
         return m
     moe = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "shared": {"ff": shared_ff, "limit": 7.0},
            "router": {"experts": experts, "identity": identity, "top": top, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}

@@ -78,7 +78,7 @@ def test_plan_names_every_tensor_and_cache_slot():
     assert parts.prefix_sharing and parts.graph_safe and parts.graph_safe_portions
     mixers = [b.parts()["mixer"] for b in parts.blocks]
     assert [m.value_mix for m in mixers] == [None, "first", "blend", "blend"]
-    assert padded_width(48, 64) == 64 and padded_width(20, 6) == 32 and padded_width(100, 7) == 128 and padded_width(130, 8) == 144
+    assert padded_width(40, 64) == 64 and padded_width(20, 6) == 32 and padded_width(100, 7) == 128 and padded_width(130, 8) == 144
 
 
 def test_plain_blocks_sinks_and_cap():

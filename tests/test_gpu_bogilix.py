@@ -64,18 +64,21 @@ def test_layer_norm_with_bias(dtype, H):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nq,nkv,dim,vdim,rot,norm", [(3, 3, 20, 6, 8, False), (6, 2, 12, 10, 0, True), (4, 1, 64, 32, 64, False),
-                                                        (8, 1, 48, 64, 0, True), (2, 2, 16, 16, 6, True)])
-def test_prepare_norms_turns_blends_and_writes_the_cache(dtype, nq, nkv, dim, vdim, rot, norm):
+                                                        (10, 2, 40, 64, 0, True), (2, 2, 16, 16, 6, True)])
+@pytest.mark.parametrize("T", [7, 300])
+def test_prepare_norms_turns_blends_and_writes_the_cache(dtype, nq, nkv, dim, vdim, rot, norm, T):
     """Whole-row norms, the rotation of a head's first numbers at positions up to a million, the blend with kept values,
     queries at the padded width with zeros behind, and keys and values where the slot mapping says (a negative slot
-    writes nothing; a page written before keeps no stale number behind the head)."""
+    writes nothing; a page written before keeps no stale number behind the head).  Seven tokens take the kernel's form
+    for few tokens (a block per head), 300 the one for many (a block per token)."""
     from sprout_lm_amd import ops
     from sprout_lm_amd.parts.sink_attention import padded_width
     rng = np.random.default_rng(nq * 100 + dim)
-    T, page, pages, eps, base = 7, 4, 6, 1e-5, 250.0
+    page, pages, eps, base = 4, 6 + T // 3, 1e-5, 250.0
     W = padded_width(dim, vdim)
     # (the bfloat16 path takes its angles in float32: off by position * 6e-8, which its tolerance holds up to some 10^4)
-    positions = np.asarray([0, 1, 5, 63, 64, 1000, 1_000_000 if dtype == torch.float32 else 20_000])
+    far = 1_000_000 if dtype == torch.float32 else 20_000
+    positions = np.concatenate([[0, 1, 5, 63, 64, 1000, far], rng.integers(0, far, T - 7)])
     cols = (nq + nkv) * dim + nkv * vdim
     proj = rounded(rng.normal(0, 1, (T, cols)), dtype)
     qn, kn = rounded(1 + rng.normal(0, 0.1, nq * dim), dtype), rounded(1 + rng.normal(0, 0.1, nkv * dim), dtype)
@@ -92,7 +95,8 @@ def test_prepare_norms_turns_blends_and_writes_the_cache(dtype, nq, nkv, dim, vd
     inv = base ** (-2.0 * np.arange(rot // 2, dtype=np.float64) / max(rot, 1))
     inv32 = inv.astype(np.float32)
     tail = (inv - inv32.astype(np.float64)).astype(np.float32)
-    slots = np.asarray([9, 2, -1, 11, 0, 23, 5], dtype=np.int32)
+    slots = rng.permutation(pages * page)[:T].astype(np.int32)
+    slots[2] = -1
     for mode in ("plain", "keep", "blend"):
         k_pool = torch.full((pages, nkv, page, W), 7.0, dtype=dtype, device=DEV)
         v_pool = torch.full((pages, nkv, W, page), 7.0, dtype=dtype, device=DEV)
@@ -184,7 +188,7 @@ def run_attention(dtype, seqs, cuts, nq, nkv, W, dim, vdim, scale, chunk, cap, s
 
 
 ATT_SHAPES = [  # nq, nkv, dim, vdim, chunk, cap, page
-    (8, 1, 48, 64, 64, 50.0, 16),     # keys narrower than values, matrix-core width 64
+    (6, 2, 40, 64, 56, 20.0, 16),     # keys narrower than values, matrix-core width 64
     (4, 2, 64, 32, 33, None, 8),      # keys wider, blocks that are no multiple of a page
     (32, 1, 16, 32, 16, 4.0, 16),     # more heads than a block of the one-query kernel holds
     (3, 3, 20, 6, 5, None, 4),        # a width only the general kernel takes
