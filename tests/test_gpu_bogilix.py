@@ -489,13 +489,15 @@ def test_replay_family(folders, name, dtype, family):
     print(f"{family} {name} {dtype}: {len(trace.steps)} steps, worst error {worst:.3e}")
 
 
-@pytest.mark.parametrize("name,page", [("general", 12), ("odd", 4), ("dense", 64)])
-def test_replay_with_other_page_sizes(folders, name, page):
+@pytest.mark.parametrize("name,page,dtype", [("general", 12, "float32"), ("odd", 4, "float32"), ("dense", 64, "float32"),
+                                             ("dense", 12, "bfloat16"), ("all_chosen", 24, "bfloat16")])
+def test_replay_with_other_page_sizes(folders, name, page, dtype):
+    """Pages of 4 to 64 tokens, also of 12 and 24 (no power of two: other prompt kernels on the bfloat16 path)."""
     requests = requests_for(name, LENGTHS[name], seed=300)
     trace = traces.mixed(requests, seed=11)
-    pool = sum(sorted(-(-len(t) // 64) * 64 for t in requests.values())[-4:])
-    results = replay(folders[name], name, "float32", trace, pool, page=page)
-    check(folders[name], "float32", requests, trace, results)
+    pool = sum(sorted(-(-len(t) // 192) * 192 for t in requests.values())[-4:])
+    results = replay(folders[name], name, dtype, trace, pool, page=page)
+    check(folders[name], dtype, requests, trace, results)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
