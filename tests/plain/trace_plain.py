@@ -20,7 +20,23 @@ import numpy as np
 from tests.plain import qwen2_plain as P
 
 
-def replay(cfg, weights, dtype: str, records, out: str) -> None:
+def plain_side(folder: str, dtype: str):
+    """(configuration, weights, logits function) of the plain implementation that config.json's architecture names."""
+    with open(os.path.join(folder, "config.json")) as f:
+        name = json.load(f).get("architecture")
+    if name == "Bogilix":
+        from tests.plain import bogilix_plain as B
+        cfg, weights = B.load_folder(folder)
+        return cfg, weights, B.forward
+    if name == "Megozen":
+        from tests.plain import megozen_plain as M
+        cfg, weights = M.load_folder(folder)
+        return cfg, weights, M.forward
+    cfg, weights = P.load_folder(folder, dtype)
+    return cfg, weights, P.forward_logits
+
+
+def replay(cfg, weights, dtype: str, records, out: str, logits_of=P.forward_logits) -> None:
     store = P.bf16_round if dtype == "bfloat16" else P.f32
     os.makedirs(out, exist_ok=True)
     history: dict[str, list[int]] = {}
@@ -33,7 +49,7 @@ def replay(cfg, weights, dtype: str, records, out: str) -> None:
                 tokens.extend(int(t) for t in item["tokens"])
                 places = [first + int(w) for w in item.get("want", [])]
                 if places:
-                    logits = P.forward_logits(weights, cfg, tokens[:max(places) + 1], store=store, rows=places)
+                    logits = logits_of(weights, cfg, tokens[:max(places) + 1], store=store, rows=places)
                     rows.extend(logits)
                     wanted += [(item["id"], p) for p in places]
             for name in record.get("end", []):
@@ -50,9 +66,9 @@ def main(argv=None) -> int:
     parser.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     parser.add_argument("--out", required=True)
     args = parser.parse_args(argv)
-    cfg, weights = P.load_folder(args.model, args.dtype)
+    cfg, weights, logits_of = plain_side(args.model, args.dtype)
     records = [json.loads(line) for line in sys.stdin if line.strip()]
-    replay(cfg, weights, args.dtype, records, args.out)
+    replay(cfg, weights, args.dtype, records, args.out, logits_of)
     return 0
 
 
